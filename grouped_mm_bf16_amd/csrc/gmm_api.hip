@@ -1,0 +1,218 @@
+// C ABI of libgrouped_mm_hip.so (declared in include/grouped_mm_hip.h): argument
+// checks, choice of kernel family, launch.  No allocation, no synchronisation,
+// no exceptions across the boundary.
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "gmm_launch.h"
+
+namespace {
+
+std::atomic<int> g_forced_path{GMM_PATH_AUTO};
+std::atomic<int> g_forced_config{-1};
+std::atomic<int> g_xcd_remap{1};
+thread_local int t_last_path = 0;
+thread_local int t_last_config = -1;
+
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_num_cus[kMaxDevices];
+
+int device_cus() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  int n = g_num_cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    n = (n / 8) * 8;  // the XCD renumbering wants a multiple of 8
+    if (n <= 0) n = 8;
+    g_num_cus[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+bool fits_i32(int64_t v) { return v >= 0 && v < (int64_t(1) << 31); }
+bool mult8(int64_t v) { return (v & 7) == 0; }
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+struct Problem {
+  GmmParams p;
+  int in_dtype, out_dtype;
+};
+
+// Decide whether the MFMA family can take the call, and with which operand layouts.
+bool mfma_eligible(const Problem& pr, GmmLayout& lay, int& align) {
+  const GmmParams& p = pr.p;
+  if (pr.in_dtype != GMM_DT_BF16) return false;
+  if (pr.out_dtype != GMM_DT_BF16 && pr.out_dtype != GMM_DT_F32) return false;
+  if (!aligned16(p.a) || !aligned16(p.b)) return false;
+  if (!mult8(p.a_sg) || !mult8(p.b_sg)) return false;
+  // A: contiguous along K (row-major) or along M (column-major)
+  if (p.a_sk == 1 && mult8(p.a_sm) && mult8(p.K)) lay.a_kc = true;
+  else if (p.a_sm == 1 && mult8(p.a_sk) && mult8(p.M) && p.M >= 8) lay.a_kc = false;
+  else return false;
+  // B: contiguous along K (column-major) or along N (row-major)
+  if (p.b_sk == 1 && mult8(p.b_sn) && mult8(p.K)) lay.b_kc = true;
+  else if (p.b_sn == 1 && mult8(p.b_sk) && mult8(p.N) && p.N >= 8) lay.b_kc = false;
+  else return false;
+  align = 1;
+  if (p.jag == GMM_JAG_M && !lay.a_kc) align = 8;
+  if (p.jag == GMM_JAG_N && !lay.b_kc) align = 8;
+  return true;
+}
+
+int run(Problem& pr, hipStream_t stream) {
+  GmmParams& p = pr.p;
+  if (!p.a || !p.b || !p.c) return GMM_ERR_BAD_ARGUMENT;
+  if (p.jag != GMM_JAG_NONE && (!p.offs || p.G < 1 || p.G >= GMM_MAX_GROUPS)) return GMM_ERR_BAD_ARGUMENT;
+  if (p.G < 0) return GMM_ERR_BAD_ARGUMENT;
+  if (pr.in_dtype < 0 || pr.in_dtype > GMM_DT_F32) return GMM_ERR_UNSUPPORTED;
+  if (pr.out_dtype != pr.in_dtype && pr.out_dtype != GMM_DT_F32) return GMM_ERR_UNSUPPORTED;
+  // Nothing to write.
+  if (p.G == 0 || p.M == 0 || p.N == 0) return GMM_OK;
+
+  const int cus = device_cus();
+  if (cus <= 0) return GMM_ERR_LAUNCH;
+
+  GmmLayout lay{};
+  int align = 1;
+  const int forced = g_forced_path.load(std::memory_order_relaxed);
+  const bool can_mfma = mfma_eligible(pr, lay, align);
+  if (forced == GMM_PATH_MFMA && !can_mfma) return GMM_ERR_UNSUPPORTED;
+  const bool use_mfma = can_mfma && forced != GMM_PATH_GENERIC;
+
+  int rc;
+  if (use_mfma) {
+    p.align = align;
+    p.xcd_remap = g_xcd_remap.load(std::memory_order_relaxed);
+    int cfg = g_forced_config.load(std::memory_order_relaxed);
+    if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = GMM_CFG_256x256;
+    rc = gmm_launch_mfma(p, lay, pr.out_dtype, cfg, cus, stream);
+    t_last_path = GMM_PATH_MFMA;
+    t_last_config = cfg;
+  } else {
+    rc = gmm_launch_generic(p, pr.in_dtype, pr.out_dtype, cus, stream);
+    t_last_path = GMM_PATH_GENERIC;
+    t_last_config = -1;
+  }
+  if (rc < 0) return GMM_ERR_UNSUPPORTED;
+  return rc == 0 ? GMM_OK : GMM_ERR_LAUNCH;
+}
+
+bool dims_ok(int64_t a, int64_t b, int64_t c) { return fits_i32(a) && fits_i32(b) && fits_i32(c); }
+
+}  // namespace
+
+extern "C" {
+
+int gmm_abi_version(void) { return GMM_ABI_VERSION; }
+
+const char* gmm_status_string(int status) {
+  switch (status) {
+    case GMM_OK: return "ok";
+    case GMM_ERR_BAD_ARGUMENT: return "bad argument (null pointer, size out of range or more than 1023 groups)";
+    case GMM_ERR_UNSUPPORTED: return "unsupported dtype combination or forced kernel family not applicable";
+    case GMM_ERR_LAUNCH: return "HIP launch failed";
+    default: return "unknown status";
+  }
+}
+
+int gmm_2d3d(const void* a, const void* b, void* out, const int32_t* offs, int32_t G, int64_t M_total,
+             int64_t N, int64_t K, int64_t a_sm, int64_t a_sk, int64_t b_sg, int64_t b_sk, int64_t b_sn,
+             int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* stream) {
+  if (!dims_ok(M_total, N, K)) return GMM_ERR_BAD_ARGUMENT;
+  Problem pr{};
+  pr.p = GmmParams{a, b, out, offs, G, GMM_JAG_M, int32_t(M_total), int32_t(N), int32_t(K), 1,
+                   0, a_sm, a_sk, b_sg, b_sk, b_sn, 0, o_sm, o_sn, 0, 0};
+  pr.in_dtype = in_dtype;
+  pr.out_dtype = out_dtype;
+  return run(pr, static_cast<hipStream_t>(stream));
+}
+
+int gmm_3d3d(const void* a, const void* b, void* out, int32_t G, int64_t M, int64_t N, int64_t K,
+             int64_t a_sg, int64_t a_sm, int64_t a_sk, int64_t b_sg, int64_t b_sk, int64_t b_sn,
+             int64_t o_sg, int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* stream) {
+  if (!dims_ok(M, N, K)) return GMM_ERR_BAD_ARGUMENT;
+  Problem pr{};
+  pr.p = GmmParams{a, b, out, nullptr, G, GMM_JAG_NONE, int32_t(M), int32_t(N), int32_t(K), 1,
+                   a_sg, a_sm, a_sk, b_sg, b_sk, b_sn, o_sg, o_sm, o_sn, 0, 0};
+  pr.in_dtype = in_dtype;
+  pr.out_dtype = out_dtype;
+  // the tile count G * tiles must fit an int32
+  if (G > 0 && M > 0 && N > 0) {
+    const int64_t tiles = int64_t(G) * ((M + 63) / 64) * ((N + 63) / 64);
+    if (!fits_i32(tiles)) return GMM_ERR_BAD_ARGUMENT;
+  }
+  return run(pr, static_cast<hipStream_t>(stream));
+}
+
+int gmm_2d2d(const void* a, const void* b, void* out, const int32_t* offs, int32_t G, int64_t M, int64_t N,
+             int64_t K_total, int64_t a_sm, int64_t a_sk, int64_t b_sk, int64_t b_sn, int64_t o_sg,
+             int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* stream) {
+  if (!dims_ok(M, N, K_total)) return GMM_ERR_BAD_ARGUMENT;
+  Problem pr{};
+  pr.p = GmmParams{a, b, out, offs, G, GMM_JAG_K, int32_t(M), int32_t(N), int32_t(K_total), 1,
+                   0, a_sm, a_sk, 0, b_sk, b_sn, o_sg, o_sm, o_sn, 0, 0};
+  pr.in_dtype = in_dtype;
+  pr.out_dtype = out_dtype;
+  return run(pr, static_cast<hipStream_t>(stream));
+}
+
+int gmm_3d2d(const void* a, const void* b, void* out, const int32_t* offs, int32_t G, int64_t M,
+             int64_t N_total, int64_t K, int64_t a_sg, int64_t a_sm, int64_t a_sk, int64_t b_sk, int64_t b_sn,
+             int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* stream) {
+  if (!dims_ok(M, N_total, K)) return GMM_ERR_BAD_ARGUMENT;
+  Problem pr{};
+  pr.p = GmmParams{a, b, out, offs, G, GMM_JAG_N, int32_t(M), int32_t(N_total), int32_t(K), 1,
+                   a_sg, a_sm, a_sk, 0, b_sk, b_sn, 0, o_sm, o_sn, 0, 0};
+  pr.in_dtype = in_dtype;
+  pr.out_dtype = out_dtype;
+  return run(pr, static_cast<hipStream_t>(stream));
+}
+
+int gmm_set_path(int path) {
+  if (path < GMM_PATH_AUTO || path > GMM_PATH_MFMA) return -1;
+  return g_forced_path.exchange(path);
+}
+int gmm_last_path(void) { return t_last_path; }
+int gmm_set_mfma_config(int config) { return g_forced_config.exchange(config); }
+int gmm_last_mfma_config(void) { return t_last_config; }
+int gmm_set_xcd_remap(int on) { return g_xcd_remap.exchange(on ? 1 : 0); }
+
+int64_t gmm_host_tile_list(const int32_t* offs_host, int32_t G, int32_t jagged, int32_t M, int32_t N, int32_t K,
+                           int32_t tile_m, int32_t tile_n, int32_t align, int32_t xcd_remap,
+                           int32_t num_workgroups, int32_t* records, int64_t capacity) {
+  if (G < 0 || jagged < 0 || jagged > 3 || tile_m <= 0 || tile_n <= 0 || align <= 0) return -GMM_ERR_BAD_ARGUMENT;
+  if (jagged != GMM_JAG_NONE && (!offs_host || G < 1 || G >= GMM_MAX_GROUPS)) return -GMM_ERR_BAD_ARGUMENT;
+  if (xcd_remap && (num_workgroups <= 0 || num_workgroups % 8)) return -GMM_ERR_BAD_ARGUMENT;
+  GmmParams p{};
+  p.offs = offs_host;
+  p.G = G; p.jag = jagged; p.M = M; p.N = N; p.K = K; p.align = align;
+  const int extent = jagged == GMM_JAG_M ? M : (jagged == GMM_JAG_N ? N : K);
+  std::vector<int32_t> cum(size_t(G) + 1, 0);
+  for (int g = 0; g < G; ++g) {
+    int lo = 0, hi = 0, tm, tn;
+    if (jagged != GMM_JAG_NONE) gmm_group_range(offs_host, g, extent, lo, hi);
+    gmm_group_grid(jagged, lo, hi, M, N, tile_m, tile_n, align, tm, tn);
+    cum[g + 1] = cum[g] + tm * tn;
+  }
+  const int total = cum[G];
+  for (int t = 0; t < total; ++t) {
+    const int tt = xcd_remap ? gmm_xcd_remap(t, total, num_workgroups) : t;
+    const int g = gmm_find_group(cum.data(), G, tt);
+    int lo = 0, hi = 0, tm, tn, mt, nt;
+    if (jagged != GMM_JAG_NONE) gmm_group_range(offs_host, g, extent, lo, hi);
+    gmm_group_grid(jagged, lo, hi, M, N, tile_m, tile_n, align, tm, tn);
+    gmm_decode_in_group(tt - cum[g], tm, tn, mt, nt);
+    const GmmTile tile = gmm_make_tile(p, g, lo, hi, mt, nt, tile_m, tile_n);
+    if (t < capacity && records) {
+      int32_t* r = records + int64_t(t) * 9;
+      r[0] = tile.g; r[1] = tile.m0; r[2] = tile.n0; r[3] = tile.m_lo; r[4] = tile.m_hi;
+      r[5] = tile.n_lo; r[6] = tile.n_hi; r[7] = tile.k_lo; r[8] = tile.k_hi;
+    }
+  }
+  return total;
+}
+
+}  // extern "C"

@@ -1,0 +1,92 @@
+// Device-side helpers shared by the gfx950 kernels: the per-workgroup tile
+// table (prefix sum of per-group tile counts kept in LDS) and dtype conversion.
+#pragma once
+#include <hip/hip_runtime.h>
+#include "gmm_sched.h"
+
+// Exclusive prefix sum of per-group tile counts into cum[0..G] (LDS), returns
+// the total.  All NT threads of the workgroup must call it; it ends with a
+// barrier.  For 3D x 3D there is no table: every group has the same grid.
+template <int NT>
+__device__ __forceinline__ int gmm_build_tile_table(const GmmParams& p, int bm, int bn, int32_t* cum) {
+  const int tid = threadIdx.x;
+  if (p.jag == GMM_JAG_NONE) return p.G * gmm_cdiv(p.M, bm) * gmm_cdiv(p.N, bn);
+
+  const int extent = p.jag == GMM_JAG_M ? p.M : (p.jag == GMM_JAG_N ? p.N : p.K);
+  for (int g = tid; g < GMM_MAX_GROUPS; g += NT) {
+    int cnt = 0;
+    if (g < p.G) {
+      int lo, hi, tm, tn;
+      gmm_group_range(p.offs, g, extent, lo, hi);
+      gmm_group_grid(p.jag, lo, hi, p.M, p.N, bm, bn, p.align, tm, tn);
+      cnt = tm * tn;
+    }
+    cum[g + 1] = cnt;
+  }
+  if (tid == 0) cum[0] = 0;
+  __syncthreads();
+  if (tid < 64) {
+    // lane l owns entries 1 + 16 l .. 16 + 16 l
+    constexpr int PER = GMM_MAX_GROUPS / 64;
+    int v[PER];
+    int run = 0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) { run += cum[1 + tid * PER + i]; v[i] = run; }
+    int incl = run;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (tid >= d) incl += up;
+    }
+    const int before = incl - run;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) cum[1 + tid * PER + i] = v[i] + before;
+  }
+  __syncthreads();
+  return cum[p.G];
+}
+
+// Linear tile id -> tile, using the table above.
+__device__ __forceinline__ GmmTile gmm_locate_tile(const GmmParams& p, const int32_t* cum, int t, int bm, int bn) {
+  int g, local, lo = 0, hi = 0, tm, tn;
+  if (p.jag == GMM_JAG_NONE) {
+    tm = gmm_cdiv(p.M, bm);
+    tn = gmm_cdiv(p.N, bn);
+    g = t / (tm * tn);
+    local = t - g * (tm * tn);
+  } else {
+    const int extent = p.jag == GMM_JAG_M ? p.M : (p.jag == GMM_JAG_N ? p.N : p.K);
+    g = gmm_find_group(cum, p.G, t);
+    local = t - cum[g];
+    gmm_group_range(p.offs, g, extent, lo, hi);
+    g = __builtin_amdgcn_readfirstlane(g);
+    local = __builtin_amdgcn_readfirstlane(local);
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    hi = __builtin_amdgcn_readfirstlane(hi);
+    gmm_group_grid(p.jag, lo, hi, p.M, p.N, bm, bn, p.align, tm, tn);
+  }
+  int mt, nt;
+  gmm_decode_in_group(local, tm, tn, mt, nt);
+  return gmm_make_tile(p, g, lo, hi, mt, nt, bm, bn);
+}
+
+// ---- element types -------------------------------------------------------- //
+struct gmm_bf16 { uint16_t bits; };
+struct gmm_f16 { _Float16 v; };
+
+__device__ __forceinline__ float gmm_to_float(gmm_bf16 x) { return __uint_as_float(uint32_t(x.bits) << 16); }
+__device__ __forceinline__ float gmm_to_float(gmm_f16 x) { return float(x.v); }
+__device__ __forceinline__ float gmm_to_float(float x) { return x; }
+
+// fp32 -> bf16 bits, round to nearest even, NaN stays NaN.
+__device__ __forceinline__ uint16_t gmm_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return uint16_t(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T gmm_from_float(float f);
+template <> __device__ __forceinline__ gmm_bf16 gmm_from_float<gmm_bf16>(float f) { return gmm_bf16{gmm_bf16_bits(f)}; }
+template <> __device__ __forceinline__ gmm_f16 gmm_from_float<gmm_f16>(float f) { return gmm_f16{_Float16(f)}; }
+template <> __device__ __forceinline__ float gmm_from_float<float>(float f) { return f; }

@@ -1,0 +1,287 @@
+// Persistent bf16 MFMA grouped GEMM for gfx950 (MI355X).
+//
+// One kernel body serves the four variants: the tile list (gmm_sched.h) turns a
+// linear tile id into a group, an origin and the row / column / contraction
+// ranges that the group owns, and the main loop is an ordinary C = A * B tile.
+//
+//   * v_mfma_f32_32x32x16_bf16, fp32 accumulators, one rounding at the end;
+//   * A and B tiles are staged in LDS as [row][64 k] with 16-byte chunks
+//     XOR-swizzled against bank conflicts, two buffers, one barrier per k-tile;
+//   * an operand that is contiguous along K is copied chunk by chunk; one that
+//     is contiguous along M or N (row-major B, column-major A) is read with
+//     16-byte loads along its contiguous dimension and transposed 8 x 8 in
+//     registers (v_perm) before it is written to LDS, so both layouts feed the
+//     same MFMA fragment reads;
+//   * stores are masked to the rows / columns the tile's own group owns, so no
+//     second "fix-up" launch is needed (the reference needs one:
+//     grouped_mm_bf16/kernels.py:363-419) and nothing outside a group is written.
+//
+// Requirements checked by the host before this family is chosen: bf16 inputs,
+// 16-byte aligned bases, leading dimensions and contiguous extents that are
+// multiples of 8 elements.
+#include "gmm_device.h"
+#include "gmm_launch.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 64;  // contraction elements per LDS tile (8 chunks of 16 bytes per row)
+
+// Swizzle of the 16-byte chunk index inside a 128-byte LDS row.
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
+
+__device__ __forceinline__ int lds_off(int row, int chunk) { return row * BK + ((chunk ^ swz(row)) << 3); }
+
+__device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
+
+// Keep elements e of a chunk with lo_e <= e < hi_e, zero the rest.
+__device__ __forceinline__ uint4 mask_chunk(uint4 v, int lo_e, int hi_e) {
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t m0 = (2 * i >= lo_e && 2 * i < hi_e) ? 0x0000ffffu : 0u;
+    const uint32_t m1 = (2 * i + 1 >= lo_e && 2 * i + 1 < hi_e) ? 0xffff0000u : 0u;
+    w[i] &= (m0 | m1);
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// ---- global -> register -> LDS staging of one ROWS x 64 operand tile ------ //
+
+// Operand contiguous along K: element (row, k) at base[row * ld + k].
+template <int ROWS, int NT>
+struct StageKC {
+  static constexpr int PER = (ROWS * 8 + NT - 1) / NT;
+  uint4 r[PER];
+
+  __device__ __forceinline__ void load(const uint16_t* base, int64_t ld, int row0, int row_ext, int kk,
+                                       int k_lo, int k_hi, bool elem_mask) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int it = 0; it < PER; ++it) {
+      const int q = it * NT + tid;
+      const int row = q >> 3, c = q & 7;
+      uint4 v = zero4();
+      if (ROWS * 8 % NT == 0 || q < ROWS * 8) {
+        const int rg = gmm_min(row0 + row, row_ext - 1);
+        const int kc = kk + c * 8;
+        if (kc < k_hi && kc + 8 > k_lo) {
+          v = *reinterpret_cast<const uint4*>(base + int64_t(rg) * ld + kc);
+          if (elem_mask) v = mask_chunk(v, k_lo - kc, k_hi - kc);
+        }
+      }
+      r[it] = v;
+    }
+  }
+
+  __device__ __forceinline__ void store(uint16_t* lds) const {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int it = 0; it < PER; ++it) {
+      const int q = it * NT + tid;
+      const int row = q >> 3, c = q & 7;
+      if (ROWS * 8 % NT == 0 || q < ROWS * 8) *reinterpret_cast<uint4*>(lds + lds_off(row, c)) = r[it];
+    }
+  }
+};
+
+// Operand contiguous along its row index (M for A, N for B): element (row, k)
+// at base[k * ld + row].  Each thread owns 8 rows x 8 k and transposes them.
+template <int ROWS, int NT>
+struct StageMC {
+  static constexpr int BLOCKS = ROWS;  // (ROWS / 8) row blocks x 8 k blocks
+  static constexpr int PER = (BLOCKS + NT - 1) / NT;
+  uint4 r[PER][8];
+
+  __device__ __forceinline__ void load(const uint16_t* base, int64_t ld, int row0, int row_ext, int kk,
+                                       int k_lo, int k_hi, bool) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int it = 0; it < PER; ++it) {
+      const int blk = it * NT + tid;
+      const int rb = blk % (ROWS / 8), kb = blk / (ROWS / 8);
+      int rg = row0 + rb * 8;
+      if (rg + 8 > row_ext) rg = row_ext - 8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int k = kk + kb * 8 + j;
+        uint4 v = zero4();
+        if ((BLOCKS % NT == 0 || blk < BLOCKS) && k >= k_lo && k < k_hi)
+          v = *reinterpret_cast<const uint4*>(base + int64_t(k) * ld + rg);
+        r[it][j] = v;
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(uint16_t* lds) const {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int it = 0; it < PER; ++it) {
+      const int blk = it * NT + tid;
+      const int rb = blk % (ROWS / 8), kb = blk / (ROWS / 8);
+      if (!(BLOCKS % NT == 0 || blk < BLOCKS)) continue;
+      const uint32_t* w = reinterpret_cast<const uint32_t*>(&r[it][0]);  // w[j * 4 + p]: k row j, word p
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        // output row i (operand row rb * 8 + i): 8 k values, two per word
+        const int pw = i >> 1;
+        const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
+        uint4 o;
+        o.x = __builtin_amdgcn_perm(w[1 * 4 + pw], w[0 * 4 + pw], sel);
+        o.y = __builtin_amdgcn_perm(w[3 * 4 + pw], w[2 * 4 + pw], sel);
+        o.z = __builtin_amdgcn_perm(w[5 * 4 + pw], w[4 * 4 + pw], sel);
+        o.w = __builtin_amdgcn_perm(w[7 * 4 + pw], w[6 * 4 + pw], sel);
+        *reinterpret_cast<uint4*>(lds + lds_off(rb * 8 + i, kb)) = o;
+      }
+    }
+  }
+};
+
+template <bool KC, int ROWS, int NT> struct StageSel { typedef StageKC<ROWS, NT> type; };
+template <int ROWS, int NT> struct StageSel<false, ROWS, NT> { typedef StageMC<ROWS, NT> type; };
+
+__device__ __forceinline__ void store_out(float* c, int64_t idx, float v) { c[idx] = v; }
+__device__ __forceinline__ void store_out(uint16_t* c, int64_t idx, float v) { c[idx] = gmm_bf16_bits(v); }
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, typename OutT>
+__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) gmm_mfma_kernel(const GmmParams p) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the MFMA tile");
+
+  __shared__ __attribute__((aligned(16))) uint16_t lds_a[2][BM * BK];
+  __shared__ __attribute__((aligned(16))) uint16_t lds_b[2][BN * BK];
+  __shared__ int32_t cum[GMM_MAX_GROUPS + 1];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+
+  const int total = gmm_build_tile_table<NT>(p, BM, BN, cum);
+  const uint16_t* __restrict__ A = static_cast<const uint16_t*>(p.a);
+  const uint16_t* __restrict__ B = static_cast<const uint16_t*>(p.b);
+  OutT* __restrict__ C = static_cast<OutT*>(p.c);
+  const int64_t a_ld = A_KC ? p.a_sm : p.a_sk;
+  const int64_t b_ld = B_KC ? p.b_sn : p.b_sk;
+
+  typename StageSel<A_KC, BM, NT>::type sa;
+  typename StageSel<B_KC, BN, NT>::type sb;
+
+  for (int t = blockIdx.x; t < total; t += gridDim.x) {
+    const int tt = p.xcd_remap ? gmm_xcd_remap(t, total, gridDim.x) : t;
+    const GmmTile tile = gmm_locate_tile(p, cum, tt, BM, BN);
+    const uint16_t* a = A + int64_t(tile.g) * p.a_sg;
+    const uint16_t* b = B + int64_t(tile.g) * p.b_sg;
+    OutT* c = C + int64_t(tile.g) * p.c_sg;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    const int k_begin = tile.k_lo & ~7;
+    const int nk = tile.k_hi > tile.k_lo ? gmm_cdiv(tile.k_hi - k_begin, BK) : 0;
+    const bool elem_mask = ((tile.k_lo | tile.k_hi) & 7) != 0;
+
+    if (nk > 0) {
+      sa.load(a, a_ld, tile.m0, p.M, k_begin, tile.k_lo, tile.k_hi, elem_mask);
+      sb.load(b, b_ld, tile.n0, p.N, k_begin, tile.k_lo, tile.k_hi, elem_mask);
+      sa.store(lds_a[0]);
+      sb.store(lds_b[0]);
+      __syncthreads();
+    }
+    for (int kt = 0; kt < nk; ++kt) {
+      const int cur = kt & 1;
+      const bool more = kt + 1 < nk;
+      if (more) {
+        const int kk = k_begin + (kt + 1) * BK;
+        sa.load(a, a_ld, tile.m0, p.M, kk, tile.k_lo, tile.k_hi, elem_mask);
+        sb.load(b, b_ld, tile.n0, p.N, kk, tile.k_lo, tile.k_hi, elem_mask);
+      }
+      const uint16_t* la = lds_a[cur];
+      const uint16_t* lb = lds_b[cur];
+#pragma unroll
+      for (int s = 0; s < BK / 16; ++s) {
+        bf16x8 af[TM], bf[TN];
+        const int chunk = 2 * s + (lane >> 5);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int row = wm * WTM + i * 32 + (lane & 31);
+          af[i] = *reinterpret_cast<const bf16x8*>(la + lds_off(row, chunk));
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int row = wn * WTN + j * 32 + (lane & 31);
+          bf[j] = *reinterpret_cast<const bf16x8*>(lb + lds_off(row, chunk));
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+      }
+      if (more) {
+        sa.store(lds_a[cur ^ 1]);
+        sb.store(lds_b[cur ^ 1]);
+      }
+      __syncthreads();
+    }
+
+    // Epilogue: lane holds, for each 32 x 32 block, column (lane % 32) and rows
+    // 8 q + 4 (lane / 32) + r for q, r in 0..3.
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = tile.m0 + wm * WTM + i * 32 + 8 * q + 4 * (lane >> 5) + r;
+          const bool row_ok = row >= tile.m_lo && row < tile.m_hi;
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            const int col = tile.n0 + wn * WTN + j * 32 + (lane & 31);
+            if (row_ok && col >= tile.n_lo && col < tile.n_hi)
+              store_out(c, int64_t(row) * p.c_sm + int64_t(col) * p.c_sn, acc[i][j][4 * q + r]);
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
+int launch_layout(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  const dim3 grid(p.num_wg), block(NT);
+  if (lay.a_kc && lay.b_kc)
+    hipLaunchKernelGGL((gmm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, true, true, OutT>), grid, block, 0, stream, p);
+  else if (lay.a_kc && !lay.b_kc)
+    hipLaunchKernelGGL((gmm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, true, false, OutT>), grid, block, 0, stream, p);
+  else if (!lay.a_kc && lay.b_kc)
+    hipLaunchKernelGGL((gmm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, false, true, OutT>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((gmm_mfma_kernel<BM, BN, WAVES_M, WAVES_N, false, false, OutT>), grid, block, 0, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
+}  // namespace
+
+void gmm_mfma_tile_shape(int config, int& bm, int& bn) {
+  (void)config;
+  bm = 256;
+  bn = 256;
+}
+
+int gmm_launch_mfma(GmmParams p, GmmLayout lay, int out_dtype, int config, int num_cus, hipStream_t stream) {
+  (void)config;
+  p.num_wg = num_cus;
+  if (out_dtype == GMM_DT_BF16) return launch_layout<256, 256, 2, 2, uint16_t>(p, lay, stream);
+  if (out_dtype == GMM_DT_F32) return launch_layout<256, 256, 2, 2, float>(p, lay, stream);
+  return -1;
+}

@@ -1,0 +1,134 @@
+// Tile scheduler shared by host and device.
+//
+// A grouped matrix multiply is a list of independent GEMM problems, one per
+// group, that differ only along one "jagged" dimension (rows for 2D x 3D,
+// columns for 3D x 2D, the contraction for 2D x 2D, none for 3D x 3D).  The
+// group boundaries live in device memory (`offs`, int32 end offsets), so the
+// number of output tiles is unknown to the host.  Every workgroup therefore
+// builds the same table on its own: per-group tile counts, their exclusive
+// prefix sum, and a decode from a linear tile id to (group, tile row, tile
+// column).  The functions here are that logic; they compile for the host too,
+// so the CPU tests can enumerate tiles exactly as the kernels do.
+//
+// Semantics followed (reference tree): the group that owns index i is the first
+// g with offs[g] > i (grouped_mm_bf16/kernels.py:162-172); empty groups own
+// nothing in 2D x 3D / 3D x 2D but still produce an all-zero slab in 2D x 2D
+// (kernels.py:276-301).
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define GMM_HD __host__ __device__ __forceinline__
+#else
+#define GMM_HD inline
+#endif
+
+enum GmmJag : int32_t { GMM_JAG_NONE = 0, GMM_JAG_M = 1, GMM_JAG_N = 2, GMM_JAG_K = 3 };
+
+constexpr int GMM_MAX_GROUPS = 1024;  // offs.numel() < 1024 is enforced by the host layer
+constexpr int GMM_BAND = 8;           // tile rows per band in the within-group tile order
+
+// Everything a kernel needs to know about one call.  Strides are in elements.
+struct GmmParams {
+  const void* a;
+  const void* b;
+  void* c;
+  const int32_t* offs;
+  int32_t G;        // number of groups (batch size for 3D x 3D)
+  int32_t jag;      // GmmJag
+  int32_t M, N, K;  // full extents; the jagged one is the total over groups
+  int32_t align;    // tile origins along the jagged dimension are rounded down to this
+  int64_t a_sg, a_sm, a_sk;
+  int64_t b_sg, b_sk, b_sn;
+  int64_t c_sg, c_sm, c_sn;
+  int32_t xcd_remap;  // 1: renumber tiles so that each XCD works on a compact block
+  int32_t num_wg;     // persistent grid size
+};
+
+GMM_HD int gmm_cdiv(int a, int b) { return (a + b - 1) / b; }
+GMM_HD int gmm_min(int a, int b) { return a < b ? a : b; }
+GMM_HD int gmm_max(int a, int b) { return a > b ? a : b; }
+
+// [lo, hi) of group g along the jagged dimension, clamped into [0, extent] and
+// made non-decreasing so that malformed offsets can never index out of bounds.
+GMM_HD void gmm_group_range(const int32_t* offs, int g, int extent, int& lo, int& hi) {
+  int s = g > 0 ? offs[g - 1] : 0;
+  int e = offs[g];
+  s = gmm_min(gmm_max(s, 0), extent);
+  e = gmm_min(gmm_max(e, 0), extent);
+  if (e < s) e = s;
+  lo = s;
+  hi = e;
+}
+
+// Tile grid of one group.  Along a jagged M or N the first tile starts at
+// lo rounded down to `align`, so that vector loads stay aligned in memory.
+GMM_HD void gmm_group_grid(int jag, int lo, int hi, int M, int N, int bm, int bn, int align,
+                           int& tiles_m, int& tiles_n) {
+  tiles_m = gmm_cdiv(M, bm);
+  tiles_n = gmm_cdiv(N, bn);
+  if (jag == GMM_JAG_M) tiles_m = hi > lo ? gmm_cdiv(hi - (lo / align) * align, bm) : 0;
+  if (jag == GMM_JAG_N) tiles_n = hi > lo ? gmm_cdiv(hi - (lo / align) * align, bn) : 0;
+}
+
+// Linear id inside a group -> (tile row, tile column).  Tile rows advance
+// fastest inside bands of GMM_BAND rows, so tiles that run at the same time
+// share a few A row panels and a few B column panels.
+GMM_HD void gmm_decode_in_group(int t, int tiles_m, int tiles_n, int& mt, int& nt) {
+  const int per_band = GMM_BAND * tiles_n;
+  const int band = t / per_band;
+  const int first = band * GMM_BAND;
+  const int rows = gmm_min(tiles_m - first, GMM_BAND);
+  const int r = t - band * per_band;
+  mt = first + r % rows;
+  nt = r / rows;
+}
+
+// Renumbering for the 8 XCDs of the chip.  Workgroup w runs on XCD w % 8 and
+// takes tiles w, w + num_wg, ...; inside every span of `num_wg` consecutive ids
+// the ids handled by one XCD are made contiguous, so that each XCD's L2 sees a
+// compact block of the tile grid.  `num_wg` must be a multiple of 8.  It is a
+// permutation of [0, total).
+GMM_HD int gmm_xcd_remap(int t, int total, int num_wg) {
+  const int span = t / num_wg;
+  const int base = span * num_wg;
+  const int len = gmm_min(total - base, num_wg);
+  const int r = t - base;
+  const int x = r & 7;
+  // ids of XCD y in this span: those r < len with r % 8 == y, i.e. (len - y + 7) / 8 of them
+  const int q = len >> 3, rem = len & 7;
+  const int start = x * q + gmm_min(x, rem);
+  return base + start + (r >> 3);
+}
+
+// Group that holds linear tile id t, given the exclusive prefix sum cum[0..G]:
+// the g with cum[g] <= t < cum[g + 1] (empty groups are skipped by construction).
+GMM_HD int gmm_find_group(const int32_t* cum, int G, int t) {
+  int lo = 0, hi = G;  // invariant: cum[lo] <= t < cum[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cum[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// One output tile, in global coordinates of the operands.
+struct GmmTile {
+  int32_t g;
+  int32_t m0, n0;        // origin of the tile
+  int32_t m_lo, m_hi;    // rows that may be stored: [m_lo, m_hi)
+  int32_t n_lo, n_hi;    // columns that may be stored
+  int32_t k_lo, k_hi;    // contraction range that contributes
+};
+
+GMM_HD GmmTile gmm_make_tile(const GmmParams& p, int g, int lo, int hi, int mt, int nt, int bm, int bn) {
+  GmmTile t;
+  t.g = g;
+  t.m0 = mt * bm; t.m_lo = 0; t.m_hi = p.M;
+  t.n0 = nt * bn; t.n_lo = 0; t.n_hi = p.N;
+  t.k_lo = 0; t.k_hi = p.K;
+  if (p.jag == GMM_JAG_M) { t.m0 += (lo / p.align) * p.align; t.m_lo = lo; t.m_hi = hi; }
+  if (p.jag == GMM_JAG_N) { t.n0 += (lo / p.align) * p.align; t.n_lo = lo; t.n_hi = hi; }
+  if (p.jag == GMM_JAG_K) { t.k_lo = lo; t.k_hi = hi; }
+  return t;
+}

@@ -1,0 +1,117 @@
+/* C ABI of libgrouped_mm_hip.so: grouped matrix multiply for AMD MI355X (gfx950).
+ *
+ * The four launchers replace, one for one, the forward launchers that the
+ * reference's host layer imports (reference grouped_mm_bf16/api.py:8-17) and
+ * calls at api.py:195, 201, 207 and 213.  Like them they write into an output the
+ * caller allocated, return without synchronising, and never allocate.
+ *
+ * Conventions
+ *   - all pointers are device pointers on the current HIP device;
+ *   - strides are in ELEMENTS, one per tensor dimension, exactly torch's
+ *     tensor.stride(); every operand may be row-major or column-major in its
+ *     last two dimensions, with any batch stride and any alignment;
+ *   - `offs` is int32[G] of non-decreasing END offsets along the jagged
+ *     dimension (the first group starts at 0); it is read on the device only;
+ *   - in_dtype / out_dtype are gmm_dtype values; out_dtype is in_dtype or
+ *     GMM_DT_F32;
+ *   - `stream` is a hipStream_t (NULL = the default stream);
+ *   - the return value is a gmm_status; nothing is thrown across the boundary.
+ *   - elements that no group owns (rows / columns at or beyond offs[G-1]) are
+ *     not written.
+ */
+#ifndef GROUPED_MM_HIP_H
+#define GROUPED_MM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GMM_ABI_VERSION 1
+
+enum gmm_status {
+  GMM_OK = 0,
+  GMM_ERR_BAD_ARGUMENT = 1, /* null pointer, negative size, G out of range, bad stride */
+  GMM_ERR_UNSUPPORTED = 2,  /* dtype combination or forced path not available */
+  GMM_ERR_LAUNCH = 3        /* the HIP runtime refused the launch */
+};
+
+enum gmm_dtype { GMM_DT_BF16 = 0, GMM_DT_F16 = 1, GMM_DT_F32 = 2 };
+
+/* Kernel families.  AUTO picks MFMA when the operands qualify (bf16, 16-byte
+ * aligned bases and leading dimensions), else GENERIC. */
+enum gmm_path { GMM_PATH_AUTO = 0, GMM_PATH_GENERIC = 1, GMM_PATH_MFMA = 2 };
+
+int gmm_abi_version(void);
+const char* gmm_status_string(int status);
+
+/* 2D x 3D: out[s_g:e_g, :] = a[s_g:e_g, :] @ b[g]   (rows jagged)
+ * a [M_total, K], b [G, K, N], out [M_total, N].
+ * Replaces grouped_mm_2d3d(mat_a, mat_b, offs, out), reference kernels.py:583-686. */
+int gmm_2d3d(const void* a, const void* b, void* out, const int32_t* offs, int32_t G,
+             int64_t M_total, int64_t N, int64_t K,
+             int64_t a_stride_m, int64_t a_stride_k,
+             int64_t b_stride_g, int64_t b_stride_k, int64_t b_stride_n,
+             int64_t out_stride_m, int64_t out_stride_n,
+             int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/* 3D x 3D: out[g] = a[g] @ b[g]
+ * a [G, M, K], b [G, K, N], out [G, M, N].
+ * Replaces grouped_mm_3d3d(mat_a, mat_b, out), reference kernels.py:524-550. */
+int gmm_3d3d(const void* a, const void* b, void* out, int32_t G,
+             int64_t M, int64_t N, int64_t K,
+             int64_t a_stride_g, int64_t a_stride_m, int64_t a_stride_k,
+             int64_t b_stride_g, int64_t b_stride_k, int64_t b_stride_n,
+             int64_t out_stride_g, int64_t out_stride_m, int64_t out_stride_n,
+             int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/* 2D x 2D: out[g] = a[:, s_g:e_g] @ b[s_g:e_g, :]   (contraction jagged; zeros if empty)
+ * a [M, K_total], b [K_total, N], out [G, M, N].
+ * Replaces grouped_mm_2d2d(mat_a, mat_b, offs, out), reference kernels.py:553-580. */
+int gmm_2d2d(const void* a, const void* b, void* out, const int32_t* offs, int32_t G,
+             int64_t M, int64_t N, int64_t K_total,
+             int64_t a_stride_m, int64_t a_stride_k,
+             int64_t b_stride_k, int64_t b_stride_n,
+             int64_t out_stride_g, int64_t out_stride_m, int64_t out_stride_n,
+             int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/* 3D x 2D: out[:, s_g:e_g] = a[g] @ b[:, s_g:e_g]   (columns jagged)
+ * a [G, M, K], b [K, N_total], out [M, N_total].
+ * Replaces grouped_mm_3d2d(mat_a, mat_b, offs, out), reference kernels.py:689-717. */
+int gmm_3d2d(const void* a, const void* b, void* out, const int32_t* offs, int32_t G,
+             int64_t M, int64_t N_total, int64_t K,
+             int64_t a_stride_g, int64_t a_stride_m, int64_t a_stride_k,
+             int64_t b_stride_k, int64_t b_stride_n,
+             int64_t out_stride_m, int64_t out_stride_n,
+             int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/* Test and tuning hooks (the reference exposes its tile knobs through environment
+ * variables read in the launcher, kernels.py:590-634; tests force tiles through
+ * them, tests/test_grouped_mm.py:388-394).  gmm_set_path forces a kernel family
+ * for later calls of this process and returns the previous setting;
+ * gmm_last_path reports the family the calling thread's last launch used
+ * (GMM_PATH_GENERIC or GMM_PATH_MFMA, 0 before any launch). */
+int gmm_set_path(int path);
+int gmm_last_path(void);
+/* Tile configuration of the MFMA family: -1 = choose from the shapes. */
+int gmm_set_mfma_config(int config);
+int gmm_last_mfma_config(void);
+/* 0 / 1: renumber tiles per XCD (default 1). */
+int gmm_set_xcd_remap(int on);
+
+/* Host-side run of the tile scheduler that the kernels execute on the device:
+ * writes up to `capacity` records of 9 int32 (group, m0, n0, m_lo, m_hi, n_lo,
+ * n_hi, k_lo, k_hi) in launch order and returns the number of tiles (which may
+ * exceed capacity), or a negative gmm_status.  `offs_host` is a HOST pointer.
+ * jagged: 0 none, 1 rows, 2 columns, 3 contraction. */
+int64_t gmm_host_tile_list(const int32_t* offs_host, int32_t G, int32_t jagged,
+                           int32_t M, int32_t N, int32_t K,
+                           int32_t tile_m, int32_t tile_n, int32_t align,
+                           int32_t xcd_remap, int32_t num_workgroups,
+                           int32_t* records, int64_t capacity);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GROUPED_MM_HIP_H */
