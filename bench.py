@@ -1,0 +1,235 @@
+#!/usr/bin/env python3
+"""Benchmark of the grouped_mm hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one forward call of ``grouped_mm`` on synthetic inputs that are already
+resident in HBM.  The default workload is the Mixtral-style 2D x 3D MoE
+up-projection (G = 8, 16384 routed rows, K = 4096, N = 14336, skewed group sizes
+from the committed fixture).  Prints ONE JSON line: useful TFLOP/s
+(2 * sum_g M_g * K * N per call), the roofline position of the kernel measured
+with HIP events on the launch stream, and -- reported only -- the same per-group
+fp32 matmul computed by the test oracle on the host CPU for a bounded sample of
+the workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "TFLOP/s + % bf16 MFMA peak, 2D×3D MoE G=8 K=4096 N=14336, 1 GPU"
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def load_sizes(key):
+    with open(os.path.join(ROOT, "tests", "golden", "group_sizes.json")) as f:
+        return json.load(f)[key]
+
+
+def make_workload(name, torch):
+    """Returns dict(a, b, offs, out, launch, flops, bytes, bound, k, desc) with CPU tensors."""
+    from grouped_mm_bf16_amd import kernels
+    g1, g2 = torch.Generator().manual_seed(1), torch.Generator().manual_seed(2)
+    bf = torch.bfloat16
+    if name == "mixtral":
+        sizes = load_sizes("mixtral_top2_g8")
+        a = torch.randn(16384, 4096, generator=g1).to(bf)
+        b = (torch.randn(8, 4096, 14336, generator=g2) * 0.02).to(bf)
+        w = dict(variant="2d3d", sizes=sizes, a=a, b=b, out_shape=(16384, 14336), out_dtype=bf,
+                 flops=2.0 * 16384 * 4096 * 14336, bound="mfma", k=4096,
+                 bytes=a.numel() * 2 + b.numel() * 2 + 16384 * 14336 * 2,
+                 desc="mixtral_moe_up_proj_2d3d_G8_M16384_K4096_N14336_skewed_top2")
+    elif name == "fine":
+        sizes = load_sizes("fine_grained_top8_g128")
+        a = torch.randn(32768, 2048, generator=g1).to(bf)
+        b = (torch.randn(128, 2048, 768, generator=g2) * 0.02).to(bf)
+        nonempty = sum(1 for s in sizes if s > 0)
+        w = dict(variant="2d3d", sizes=sizes, a=a, b=b, out_shape=(32768, 768), out_dtype=bf,
+                 flops=2.0 * 32768 * 2048 * 768, bound="hbm", k=2048,
+                 bytes=a.numel() * 2 + nonempty * 2048 * 768 * 2 + 32768 * 768 * 2,
+                 desc="fine_grained_moe_2d3d_G128_M32768_K2048_N768_top8")
+    elif name in ("batched", "batched_colmajor"):
+        a = torch.randn(32, 1024, 1024, generator=g1).to(bf)
+        b = (torch.randn(32, 1024, 4096, generator=g2) * 0.02).to(bf)
+        w = dict(variant="3d3d", sizes=None, a=a, b=b, out_shape=(32, 1024, 4096), out_dtype=bf,
+                 flops=2.0 * 32 * 1024 * 1024 * 4096, bound="mfma", k=1024,
+                 bytes=a.numel() * 2 + b.numel() * 2 + 32 * 1024 * 4096 * 2,
+                 desc="batched_3d3d_G32_M1024_K1024_N4096" + ("_Bcolmajor" if name.endswith("colmajor") else ""),
+                 b_col=name.endswith("colmajor"))
+    elif name == "kgrouped":
+        sizes = load_sizes("mixtral_top2_g8")
+        a = torch.randn(4096, 16384, generator=g1).to(bf)
+        b = torch.randn(16384, 14336, generator=g2).to(bf)
+        w = dict(variant="2d2d", sizes=sizes, a=a, b=b, out_shape=(8, 4096, 14336), out_dtype=torch.float32,
+                 flops=2.0 * 4096 * 16384 * 14336, bound="mfma", k=16384,
+                 bytes=a.numel() * 2 + b.numel() * 2 + 8 * 4096 * 14336 * 4,
+                 desc="k_grouped_weight_grad_2d2d_G8_M4096_Ktotal16384_N14336_fp32out")
+    else:
+        raise SystemExit(f"unknown workload {name}")
+    w["launch"] = {"2d3d": kernels.grouped_mm_2d3d, "3d3d": kernels.grouped_mm_3d3d,
+                   "2d2d": kernels.grouped_mm_2d2d, "3d2d": kernels.grouped_mm_3d2d}[w["variant"]]
+    return w
+
+
+def cpu_baseline(w, torch, budget_s=15.0):
+    """The oracle (per-group fp32 torch.matmul on the host) on a bounded sample."""
+    from oracle import grouped_mm_oracle as oracle
+    threads = os.cpu_count() or 1
+    try:
+        threads = min(threads, len(os.sched_getaffinity(0)))
+    except AttributeError:
+        pass
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        threads = min(threads, int(env))
+    torch.set_num_threads(threads)
+    a, b, sizes = w["a"], w["b"], w["sizes"]
+    if w["variant"] == "2d3d":
+        ranges = oracle.group_ranges(torch.tensor(sizes).cumsum(0).tolist())
+        order = sorted(range(len(sizes)), key=lambda g: sizes[g])  # small groups first
+        order = [g for g in order if sizes[g] > 0]
+        K, N = a.shape[1], b.shape[2]
+
+        def run(groups):
+            af = [a[ranges[g][0]:ranges[g][1]].float() for g in groups]
+            bfl = [b[g].float() for g in groups]
+            t0 = time.perf_counter()
+            for x, y in zip(af, bfl):
+                torch.matmul(x, y)
+            return time.perf_counter() - t0, sum(2.0 * x.shape[0] * K * N for x in af)
+
+        # probe with the median group, then take as many groups as fit the budget
+        probe = [order[len(order) // 2]]
+        run(probe)
+        t, fl = run(probe)
+        rate = fl / max(t, 1e-9)
+        chosen, work = [], 0.0
+        for g in order[::-1]:
+            f = 2.0 * sizes[g] * K * N
+            if chosen and (work + f) / rate > budget_s:
+                continue
+            chosen.append(g)
+            work += f
+        t, fl = run(chosen)
+        sample = f"groups {sorted(chosen)} of {len(sizes)} ({fl / w['flops'] * 100:.0f}% of the step's FLOPs), 1 timed run after a probe"
+    else:
+        # batched / K-grouped: a slab of the first group
+        if w["variant"] == "3d3d":
+            x, y = a[0].float(), b[0].float()
+        else:
+            e = sizes[0]
+            x, y = a[:, :e].float(), b[:e].float()
+        torch.matmul(x[:64], y)
+        t0 = time.perf_counter()
+        torch.matmul(x, y)
+        t = time.perf_counter() - t0
+        fl = 2.0 * x.shape[0] * x.shape[1] * y.shape[1]
+        sample = f"first group only ({fl / w['flops'] * 100:.0f}% of the step's FLOPs), 1 timed run"
+    return {"value": round(fl / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": sample, "seconds": round(t, 3)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="mixtral",
+                    choices=["mixtral", "fine", "batched", "batched_colmajor", "kgrouped"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--path", default="auto", choices=["auto", "mfma", "generic"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: grouped_mm has no multi-GPU path in this build "
+                         "(run with --gpus 1)")
+
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
+    from grouped_mm_bf16_amd import kernels
+    from oracle import grouped_mm_oracle as oracle
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = make_workload(args.workload, torch)
+    a, b = w["a"].to(dev), w["b"].to(dev)
+    if w.get("b_col"):
+        b = b.transpose(-2, -1).contiguous().transpose(-2, -1)
+    offs = None
+    if w["sizes"] is not None:
+        offs = torch.tensor(w["sizes"], dtype=torch.int64).cumsum(0).to(torch.int32).to(dev)
+    out = torch.empty(w["out_shape"], device=dev, dtype=w["out_dtype"])
+
+    def step():
+        if offs is None:
+            w["launch"](a, b, out)
+        else:
+            w["launch"](a, b, offs, out)
+
+    with kernels.forced_path(args.path):
+        # parity spot-check on the tensors that are about to be timed
+        step()
+        torch.cuda.synchronize()
+        if w["variant"] == "2d3d":
+            ol = offs.cpu().tolist()
+            for r in (0, ol[0] - 1 if ol[0] > 0 else 0, ol[-1] - 1):
+                g = oracle.upper_bound(ol, r)
+                want = (w["a"][r:r + 1].float() @ w["b"][g].float()).to(out.dtype)
+                oracle.assert_close(out[r:r + 1].cpu(), want, w["k"], what=f"bench parity row {r}")
+        path = kernels.last_path()
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        # whole-job wall clock over exactly `steps` steps
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        # per-launch kernel time: HIP events on the launch stream around each step
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+               for _ in range(args.steps)]
+        for e0, e1 in evs:
+            e0.record()
+            step()
+            e1.record()
+        torch.cuda.synchronize()
+        k_ms = [e0.elapsed_time(e1) for e0, e1 in evs]
+
+    ms_per_step = wall / args.steps * 1e3
+    tflops = w["flops"] / (ms_per_step * 1e-3) / 1e12
+    k_avg = statistics.mean(k_ms)
+    if w["bound"] == "mfma":
+        achieved, peak, unit = w["flops"] / (k_avg * 1e-3) / 1e12, PEAK_BF16_TFLOPS, "TFLOP/s"
+    else:
+        achieved, peak, unit = w["bytes"] / (k_avg * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+    rec = {
+        "metric": METRIC, "value": round(tflops, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": w["desc"], "kernel_family": path,
+                   "pct_bf16_mfma_peak": round(tflops / PEAK_BF16_TFLOPS * 100, 2)},
+        "roofline": {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(k_ms), 4),
+                     "kernel_ms_median": round(statistics.median(k_ms), 4),
+                     "algorithmic_flops": w["flops"], "algorithmic_bytes": w["bytes"]},
+    }
+    if not args.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline(w, torch)
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,129 @@
+"""Launchers: the same four names and argument meaning as the forward launchers
+of the reference (``grouped_mm_bf16/kernels.py:524-717``) -- each writes into a
+caller-allocated ``out`` and returns None -- but they hand raw pointers, sizes
+and strides to the gfx950 kernels behind the C ABI instead of JIT-compiling
+Triton.  ``out.dtype`` selects the epilogue (input dtype or float32), as the
+reference's ``OUT_DTYPE=_as_tl_dtype(out.dtype)`` does.
+
+The launch itself is registered as the torch custom op
+``grouped_mm_bf16_amd::launch`` (mutating ``out``) so that it is visible to
+torch's dispatcher and tracing; it runs on the current stream of the operands'
+device and never synchronises.
+"""
+from __future__ import annotations
+
+import contextlib
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.bfloat16: _lib.DT_BF16, torch.float16: _lib.DT_F16, torch.float32: _lib.DT_F32}
+
+V_2D3D, V_3D3D, V_2D2D, V_3D2D = 0, 1, 2, 3
+
+
+def _dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise RuntimeError(f"Unsupported dtype: {dtype}") from None
+
+
+def _require_gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("grouped_mm_bf16 is GPU-only (CUDA/HIP); CPU tensors are not supported")
+
+
+@torch.library.custom_op("grouped_mm_bf16_amd::launch", mutates_args=("out",))
+def _launch(variant: int, a: torch.Tensor, b: torch.Tensor, offs: Optional[torch.Tensor],
+            out: torch.Tensor) -> None:
+    lib = _lib.load()
+    _require_gpu(a, b, offs, out)
+    in_dt, out_dt = _dtype_code(a.dtype), _dtype_code(out.dtype)
+    with torch.cuda.device(a.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        pa, pb, po = a.data_ptr(), b.data_ptr(), out.data_ptr()
+        poffs = offs.data_ptr() if offs is not None else None
+        if variant == V_2D3D:
+            rc = lib.gmm_2d3d(pa, pb, po, poffs, offs.numel(), a.size(0), b.size(2), a.size(1),
+                              a.stride(0), a.stride(1), b.stride(0), b.stride(1), b.stride(2),
+                              out.stride(0), out.stride(1), in_dt, out_dt, stream)
+        elif variant == V_3D3D:
+            rc = lib.gmm_3d3d(pa, pb, po, a.size(0), a.size(1), b.size(2), a.size(2),
+                              a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1), b.stride(2),
+                              out.stride(0), out.stride(1), out.stride(2), in_dt, out_dt, stream)
+        elif variant == V_2D2D:
+            rc = lib.gmm_2d2d(pa, pb, po, poffs, offs.numel(), a.size(0), b.size(1), a.size(1),
+                              a.stride(0), a.stride(1), b.stride(0), b.stride(1),
+                              out.stride(0), out.stride(1), out.stride(2), in_dt, out_dt, stream)
+        elif variant == V_3D2D:
+            rc = lib.gmm_3d2d(pa, pb, po, poffs, offs.numel(), a.size(1), b.size(1), a.size(2),
+                              a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1),
+                              out.stride(0), out.stride(1), in_dt, out_dt, stream)
+        else:
+            raise RuntimeError(f"unknown variant {variant}")
+    _lib.check(rc, "grouped_mm launch")
+
+
+def grouped_mm_3d3d(mat_a: torch.Tensor, mat_b: torch.Tensor, out: torch.Tensor) -> None:
+    """out[g] = mat_a[g] @ mat_b[g]  (reference ``kernels.py:524-550``)."""
+    if mat_a.size(0) != mat_b.size(0):
+        raise RuntimeError("batched dimension has to match")
+    _launch(V_3D3D, mat_a, mat_b, None, out)
+
+
+def grouped_mm_2d2d(mat_a: torch.Tensor, mat_b: torch.Tensor, offs: torch.Tensor, out: torch.Tensor) -> None:
+    """out[g] = mat_a[:, s_g:e_g] @ mat_b[s_g:e_g, :], zeros for an empty group
+    (reference ``kernels.py:553-580``)."""
+    _launch(V_2D2D, mat_a, mat_b, offs, out)
+
+
+def grouped_mm_2d3d(mat_a: torch.Tensor, mat_b: torch.Tensor, offs: torch.Tensor, out: torch.Tensor) -> None:
+    """out[s_g:e_g] = mat_a[s_g:e_g] @ mat_b[g]  (reference ``kernels.py:583-686``)."""
+    if offs.numel() != mat_b.size(0):
+        raise RuntimeError("matrix batch sizes have to match")
+    if mat_a.size(0) == 0 or mat_b.size(2) == 0:
+        return
+    _launch(V_2D3D, mat_a, mat_b, offs, out)
+
+
+def grouped_mm_3d2d(mat_a: torch.Tensor, mat_b: torch.Tensor, offs: torch.Tensor, out: torch.Tensor) -> None:
+    """out[:, s_g:e_g] = mat_a[g] @ mat_b[:, s_g:e_g]  (reference ``kernels.py:689-717``)."""
+    if offs.numel() != mat_a.size(0):
+        raise RuntimeError("matrix batch sizes have to match")
+    _launch(V_3D2D, mat_a, mat_b, offs, out)
+
+
+# ---- test / tuning hooks ---------------------------------------------------- #
+@contextlib.contextmanager
+def forced_path(path: str):
+    """Force a kernel family ("auto", "generic" or "mfma") inside the block.
+
+    The reference's tests force tile sizes through environment variables
+    (``tests/test_grouped_mm.py:388-394``); this is the equivalent hook here.
+    """
+    code = {"auto": _lib.PATH_AUTO, "generic": _lib.PATH_GENERIC, "mfma": _lib.PATH_MFMA}[path]
+    lib = _lib.load()
+    prev = lib.gmm_set_path(code)
+    try:
+        yield
+    finally:
+        lib.gmm_set_path(prev)
+
+
+@contextlib.contextmanager
+def forced_mfma_config(config: int):
+    lib = _lib.load()
+    prev = lib.gmm_set_mfma_config(config)
+    try:
+        yield
+    finally:
+        lib.gmm_set_mfma_config(prev)
+
+
+def last_path() -> str:
+    """Kernel family used by this thread's last launch: "generic", "mfma" or "none"."""
+    return {0: "none", _lib.PATH_GENERIC: "generic", _lib.PATH_MFMA: "mfma"}[_lib.load().gmm_last_path()]

@@ -1,0 +1,407 @@
+"""Parity of the HIP path with the CPU oracle, on a real MI355X.
+
+Shapes, size lists and tolerances restate the reference's own test matrix
+(reference tests/test_grouped_mm.py: :19 3Dx3D, :32 2Dx3D, :70 2Dx2D, :109 3Dx2D,
+:356-370 the seven boundary lists, :661-747 the 1023-group cases) and add the
+benchmark workloads.  Tolerance: rtol 1.6e-2, atol 1e-2 * sqrt(K / 64) against
+the fp32 oracle; which elements are written is checked exactly (NaN poisoning).
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from grouped_mm_bf16_amd import grouped_mm
+from grouped_mm_bf16_amd import kernels as K_
+from oracle import grouped_mm_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def offs_of(sizes):
+    return torch.tensor(sizes, dtype=torch.int64).cumsum(0).to(torch.int32)
+
+
+def rnd(gen, *shape, dtype=torch.bfloat16, scale=1.0):
+    return (torch.randn(*shape, generator=gen) * scale).to(dtype)
+
+
+def run_poisoned(variant_fn, a, b, offs, shape, dtype):
+    """Launch into a NaN-filled output so unwritten elements stay visible."""
+    out = torch.full(shape, float("nan"), device=DEV, dtype=dtype)
+    if offs is None:
+        variant_fn(a.to(DEV), b.to(DEV), out)
+    else:
+        variant_fn(a.to(DEV), b.to(DEV), offs.to(DEV), out)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def check(out, a, b, offs, k, path=None):
+    want = oracle.grouped_mm(a, b, offs, out_dtype=out.dtype)
+    got = out.cpu()
+    # structure: exactly the owned elements are written
+    assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs"
+    oracle.assert_close(got, want, k)
+    if path is not None:
+        assert K_.last_path() == path
+
+
+# ------------------------------------------------------------------ golden fixtures
+@pytest.mark.parametrize("name,a_shape,b_shape", [
+    ("2d3d", (32, 64), (6, 64, 48)), ("3d3d", (4, 32, 64), (4, 64, 48)),
+    ("2d2d", (16, 32), (32, 24)), ("3d2d", (5, 32, 48), (48, 32)),
+])
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+def test_golden_vectors(golden_dir, name, a_shape, b_shape, path):
+    z = np.load(os.path.join(golden_dir, "small_cases.npz"))
+    bits = lambda arr, shape: torch.from_numpy(arr.astype(np.int16)).view(torch.bfloat16).reshape(shape)
+    a, b = bits(z[f"a_{name}"], a_shape), bits(z[f"b_{name}"], b_shape)
+    offs = torch.from_numpy(z[f"offs_{name}"]) if f"offs_{name}" in z else None
+    with K_.forced_path(path):
+        got = grouped_mm(a.to(DEV), b.to(DEV), offs=None if offs is None else offs.to(DEV)).cpu()
+    want = bits(z[f"out_{name}"], got.shape)
+    own = ~torch.isnan(oracle.grouped_mm(a, b, offs).float())
+    oracle.assert_close(got[own], want[own], a.shape[-1])
+    assert K_.last_path() == path
+
+
+# ------------------------------------------------------------------ the reference's basic cases
+@pytest.mark.parametrize("path", ["auto", "generic"])
+def test_3d3d_bf16(path):
+    gen = torch.Generator().manual_seed(0)
+    a, b = rnd(gen, 4, 32, 64), rnd(gen, 4, 64, 48)
+    with K_.forced_path(path):
+        out = run_poisoned(K_.grouped_mm_3d3d, a, b, None, (4, 32, 48), torch.bfloat16)
+    check(out, a, b, None, 64)
+
+
+@pytest.mark.parametrize("path", ["auto", "generic"])
+def test_2d3d_bf16_with_empty_groups(path):
+    gen = torch.Generator().manual_seed(1)
+    sizes = [0, 7, 1, 13, 0, 11]
+    a, b = rnd(gen, 32, 32), rnd(gen, 6, 32, 40)
+    with K_.forced_path(path):
+        out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs_of(sizes), (32, 40), torch.bfloat16)
+    check(out, a, b, offs_of(sizes), 32)
+
+
+@pytest.mark.parametrize("path", ["auto", "generic"])
+def test_2d2d_bf16_empty_group_is_zero(path):
+    gen = torch.Generator().manual_seed(2)
+    sizes = [7, 0, 1, 13, 11]
+    a, b = rnd(gen, 16, 32), rnd(gen, 32, 24)
+    with K_.forced_path(path):
+        out = run_poisoned(K_.grouped_mm_2d2d, a, b, offs_of(sizes), (5, 16, 24), torch.bfloat16)
+    check(out, a, b, offs_of(sizes), 13)
+    assert (out[1] == 0).all() and not torch.isnan(out.float()).any()
+
+
+@pytest.mark.parametrize("path", ["auto", "generic"])
+def test_3d2d_bf16(path):
+    gen = torch.Generator().manual_seed(3)
+    sizes = [7, 0, 1, 13, 11]
+    a, b = rnd(gen, 5, 32, 48), rnd(gen, 48, 32)
+    with K_.forced_path(path):
+        out = run_poisoned(K_.grouped_mm_3d2d, a, b, offs_of(sizes), (32, 32), torch.bfloat16)
+    check(out, a, b, offs_of(sizes), 48)
+
+
+BOUNDARY_LISTS = [
+    [32, 32, 32], [10, 10, 10, 2], [31, 1, 31], [40, 30, 10, 7], [32, 16, 0, 0, 0],
+    [1, 0, 1, 0, 1, 0, 1, 0, 1, 0, 1, 0], [5, 0, 7, 0, 3, 9],
+]
+
+
+@pytest.mark.parametrize("sizes", BOUNDARY_LISTS)
+def test_2d3d_boundary_lists_unaligned_shapes(sizes):
+    """K = 33, N = 29: no 16-byte alignment anywhere, so the generic family runs."""
+    gen = torch.Generator().manual_seed(sum(sizes))
+    m = sum(sizes)
+    a, b = rnd(gen, m, 33), rnd(gen, len(sizes), 33, 29)
+    out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs_of(sizes), (m, 29), torch.bfloat16)
+    check(out, a, b, offs_of(sizes), 33, path="generic")
+
+
+@pytest.mark.parametrize("sizes", BOUNDARY_LISTS + [[300, 0, 1, 255, 256, 257, 33], [256, 256], [257, 255, 512]])
+@pytest.mark.parametrize("b_col", [False, True])
+def test_2d3d_boundary_lists_mfma(sizes, b_col):
+    """Same lists on aligned K / N so that the MFMA family and its 256-row tiles run."""
+    gen = torch.Generator().manual_seed(sum(sizes) + 1)
+    m = sum(sizes)
+    a, b = rnd(gen, m, 72), rnd(gen, len(sizes), 72, 264)
+    bd = b.to(DEV)
+    if b_col:
+        bd = bd.transpose(1, 2).contiguous().transpose(1, 2)
+    out = torch.full((m, 264), float("nan"), device=DEV, dtype=torch.bfloat16)
+    K_.grouped_mm_2d3d(a.to(DEV), bd, offs_of(sizes).to(DEV), out)
+    check(out, a, b, offs_of(sizes), 72, path="mfma")
+
+
+def test_rows_past_the_last_offset_are_not_written():
+    gen = torch.Generator().manual_seed(5)
+    a, b = rnd(gen, 40, 64), rnd(gen, 2, 64, 48)
+    offs = offs_of([9, 14])  # rows 23..39 belong to nobody
+    for path in ("mfma", "generic"):
+        with K_.forced_path(path):
+            out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs, (40, 48), torch.bfloat16)
+        check(out, a, b, offs, 64, path=path)
+        assert torch.isnan(out[23:].float()).all()
+
+
+# ------------------------------------------------------------------ operand layouts
+@pytest.mark.parametrize("a_col", [False, True])
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("variant", ["2d3d", "3d3d", "2d2d", "3d2d"])
+def test_all_layouts_all_variants_mfma(variant, a_col, b_col):
+    gen = torch.Generator().manual_seed(17)
+    sizes = [77, 0, 1, 130, 64, 200]  # sum 472
+    offs = offs_of(sizes)
+    G = len(sizes)
+    if variant == "2d3d":
+        a, b, shape, k, fn = rnd(gen, 472, 136), rnd(gen, G, 136, 264), (472, 264), 136, K_.grouped_mm_2d3d
+    elif variant == "3d3d":
+        a, b, shape, k, fn, offs = rnd(gen, 3, 304, 136), rnd(gen, 3, 136, 264), (3, 304, 264), 136, K_.grouped_mm_3d3d, None
+    elif variant == "2d2d":
+        a, b, shape, k, fn = rnd(gen, 264, 472), rnd(gen, 472, 272), (G, 264, 272), 200, K_.grouped_mm_2d2d
+    else:
+        a, b, shape, k, fn = rnd(gen, G, 264, 136), rnd(gen, 136, 472), (264, 472), 136, K_.grouped_mm_3d2d
+    ad, bd = a.to(DEV), b.to(DEV)
+    if a_col:
+        ad = ad.transpose(-2, -1).contiguous().transpose(-2, -1)
+    if b_col:
+        bd = bd.transpose(-2, -1).contiguous().transpose(-2, -1)
+    out = torch.full(shape, float("nan"), device=DEV, dtype=torch.bfloat16)
+    if offs is None:
+        fn(ad, bd, out)
+    else:
+        fn(ad, bd, offs.to(DEV), out)
+    check(out, a, b, offs, k, path="mfma")
+
+
+def test_row_major_and_column_major_b_agree_bit_for_bit():
+    gen = torch.Generator().manual_seed(19)
+    a, b = rnd(gen, 4, 256, 512).to(DEV), rnd(gen, 4, 512, 256, scale=0.02).to(DEV)
+    b_col = b.transpose(1, 2).contiguous().transpose(1, 2)
+    assert torch.equal(grouped_mm(a, b).view(torch.int16), grouped_mm(a, b_col).view(torch.int16))
+
+
+# ------------------------------------------------------------------ dtypes
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-4), (torch.float16, 2e-2)])
+def test_fp32_and_fp16_inputs(dtype, tol):
+    gen = torch.Generator().manual_seed(23)
+    sizes = [0, 7, 1, 13, 0, 11]
+    a, b = rnd(gen, 32, 29, dtype=dtype), rnd(gen, 6, 29, 31, dtype=dtype)
+    got = grouped_mm(a.to(DEV), b.to(DEV), offs=offs_of(sizes).to(DEV)).cpu()
+    assert got.dtype == dtype and K_.last_path() == "generic"
+    want = oracle.grouped_mm(a, b, offs_of(sizes))
+    torch.testing.assert_close(got, want, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("variant", ["2d3d", "3d2d", "2d2d"])
+def test_1023_groups_fp32(variant):
+    """G = 1023, sizes alternate 1, 0 with a trailing empty group (reference tests :661-747)."""
+    gen = torch.Generator().manual_seed(29)
+    sizes = [1 if i % 2 == 0 else 0 for i in range(1023)]
+    sizes[-1] = 0
+    tot, offs = sum(sizes), offs_of(sizes)
+    if variant == "2d3d":
+        a, b = rnd(gen, tot, 8, dtype=torch.float32), rnd(gen, 1023, 8, 8, dtype=torch.float32)
+    elif variant == "3d2d":
+        a, b = rnd(gen, 1023, 4, 8, dtype=torch.float32), rnd(gen, 8, tot, dtype=torch.float32)
+    else:
+        a, b = rnd(gen, 4, tot, dtype=torch.float32), rnd(gen, tot, 8, dtype=torch.float32)
+    got = grouped_mm(a.to(DEV), b.to(DEV), offs=offs.to(DEV)).cpu()
+    want = oracle.grouped_mm(a, b, offs)
+    torch.testing.assert_close(got, want, rtol=3e-4, atol=3e-4)
+
+
+def test_1023_groups_bf16_mfma():
+    gen = torch.Generator().manual_seed(31)
+    sizes = [3 if i % 2 == 0 else 0 for i in range(1023)]
+    sizes[-1] = 0
+    tot, offs = sum(sizes), offs_of(sizes)
+    a, b = rnd(gen, tot, 64), rnd(gen, 1023, 64, 16)
+    out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs, (tot, 16), torch.bfloat16)
+    check(out, a, b, offs, 64, path="mfma")
+
+
+def test_fp32_epilogue_for_bf16_inputs_through_the_launcher():
+    """The public function keeps the reference's dtype rule; the launcher honours out.dtype."""
+    gen = torch.Generator().manual_seed(37)
+    sizes = [40, 0, 88]
+    a, b = rnd(gen, 64, 128), rnd(gen, 128, 72)
+    out = run_poisoned(K_.grouped_mm_2d2d, a, b, offs_of(sizes), (3, 64, 72), torch.float32)
+    want = oracle.grouped_mm(a, b, offs_of(sizes), out_dtype=torch.float32)
+    torch.testing.assert_close(out, want, rtol=1e-4, atol=1e-4)
+    with pytest.raises(RuntimeError, match="output dtype must match"):
+        grouped_mm(a.to(DEV), b.to(DEV), offs=offs_of(sizes).to(DEV), out_dtype=torch.float32)
+
+
+# ------------------------------------------------------------------ host rules on real tensors
+def test_rules_on_gpu_tensors_and_shortcuts():
+    a = torch.randn(8, 16, device=DEV, dtype=torch.bfloat16)
+    b = torch.randn(2, 16, 8, device=DEV, dtype=torch.bfloat16)
+    offs = torch.tensor([3, 8], device=DEV, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="Bias not supported yet"):
+        grouped_mm(a, b, offs=offs, bias=torch.zeros(8, device=DEV))
+    with pytest.raises(RuntimeError, match="CPU offs are not supported"):
+        grouped_mm(a, b, offs=offs.cpu())
+    with pytest.raises(RuntimeError, match="Have to provide offsets"):
+        grouped_mm(a, b)
+    with pytest.raises(RuntimeError, match="matrix batch sizes have to match"):
+        grouped_mm(a, b, offs=torch.tensor([3, 5, 8], device=DEV, dtype=torch.int32))
+    # K == 0 gives zeros, an empty output comes back empty (reference api.py:188-212)
+    z = grouped_mm(a[:, :0], b[:, :0, :], offs=offs)
+    assert z.shape == (8, 8) and (z == 0).all()
+    e = grouped_mm(a[:0], b, offs=torch.zeros(2, device=DEV, dtype=torch.int32))
+    assert e.shape == (0, 8)
+    # positional and keyword call styles
+    assert torch.equal(grouped_mm(a, b, offs), grouped_mm(mat_a=a, mat_b=b, offs=offs))
+
+
+def test_runs_on_the_current_stream_without_sync():
+    gen = torch.Generator().manual_seed(41)
+    a, b = rnd(gen, 512, 256).to(DEV), rnd(gen, 4, 256, 256).to(DEV)
+    offs = offs_of([100, 0, 300, 112]).to(DEV)
+    ref = grouped_mm(a, b, offs=offs)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        got = grouped_mm(a, b, offs=offs)
+    s.synchronize()
+    assert torch.equal(got, ref)
+
+
+# ------------------------------------------------------------------ backward (composition of forwards)
+@pytest.mark.parametrize("variant", ["2d3d", "3d3d", "2d2d", "3d2d"])
+def test_backward_fp32_matches_autograd_of_the_loop(variant):
+    gen = torch.Generator().manual_seed(43)
+    sizes = [0, 7, 1, 13, 0, 11]
+    G, tot, offs = len(sizes), sum(sizes), offs_of(sizes)
+    f32 = torch.float32
+    if variant == "2d3d":
+        a, b = rnd(gen, tot, 29, dtype=f32), rnd(gen, G, 29, 31, dtype=f32)
+    elif variant == "3d3d":
+        a, b, offs = rnd(gen, 3, 17, 19, dtype=f32), rnd(gen, 3, 19, 23, dtype=f32), None
+    elif variant == "2d2d":
+        a, b = rnd(gen, 19, tot, dtype=f32), rnd(gen, tot, 21, dtype=f32)
+    else:
+        a, b = rnd(gen, G, 23, 17, dtype=f32), rnd(gen, 17, tot, dtype=f32)
+    ad, bd = a.to(DEV).requires_grad_(), b.to(DEV).requires_grad_()
+    out = grouped_mm(ad, bd, offs=None if offs is None else offs.to(DEV))
+    w = torch.randn(out.shape, generator=gen)
+    (out * w.to(DEV)).sum().backward()
+
+    ar, br = a.clone().requires_grad_(), b.clone().requires_grad_()
+    rng = oracle.group_ranges(offs.tolist()) if offs is not None else None
+    if variant == "2d3d":
+        ref = torch.cat([ar[s:e] @ br[g] for g, (s, e) in enumerate(rng)])
+    elif variant == "3d3d":
+        ref = torch.bmm(ar, br)
+    elif variant == "2d2d":
+        ref = torch.stack([ar[:, s:e] @ br[s:e] for (s, e) in rng])
+    else:
+        ref = torch.cat([ar[g] @ br[:, s:e] for g, (s, e) in enumerate(rng)], dim=1)
+    (ref * w).sum().backward()
+    torch.testing.assert_close(out.detach().cpu(), ref.detach(), rtol=3e-4, atol=3e-4)
+    torch.testing.assert_close(ad.grad.cpu(), ar.grad, rtol=8e-4, atol=8e-4)
+    torch.testing.assert_close(bd.grad.cpu(), br.grad, rtol=8e-4, atol=8e-4)
+
+
+# ------------------------------------------------------------------ benchmark workloads, full size
+def _sizes(golden_dir, key):
+    with open(os.path.join(golden_dir, "group_sizes.json")) as f:
+        return json.load(f)[key]
+
+
+def _sampled_check(out, a, b, offs_list, k, rows, cols=slice(None)):
+    """Oracle on a sample of rows of a big 2D x 3D result."""
+    ranges = oracle.group_ranges(offs_list)
+    for r in rows:
+        g = oracle.upper_bound(offs_list, r)
+        s, e = ranges[g]
+        assert s <= r < e
+        want = (a[r:r + 1].float() @ b[g].float()).to(out.dtype)
+        oracle.assert_close(out[r:r + 1].cpu(), want, k, what=f"row {r} group {g}")
+
+
+def test_mixtral_up_projection_full_size(golden_dir):
+    sizes = _sizes(golden_dir, "mixtral_top2_g8")
+    offs = offs_of(sizes)
+    gen = torch.Generator().manual_seed(1)
+    a = rnd(gen, 16384, 4096)
+    b = rnd(torch.Generator().manual_seed(2), 8, 4096, 14336, scale=0.02)
+    ad, bd = a.to(DEV), b.to(DEV)
+    out = grouped_mm(ad, bd, offs=offs.to(DEV))
+    assert K_.last_path() == "mfma"
+    ol = offs.tolist()
+    rows = sorted({0, 1, 255, 256, 16383, *ol[:-1], *[o - 1 for o in ol], *range(4800, 4830, 7), *range(0, 16384, 1999)})
+    _sampled_check(out, a, b, ol, 4096, rows)
+    # size-independent properties: splitting every group in two (same weights) and
+    # permuting the groups must reproduce the same rows bit for bit
+    halves, idx = [], []
+    for g, s in enumerate(sizes):
+        halves += [s // 2, s - s // 2]
+        idx += [g, g]
+    out2 = grouped_mm(ad, bd[idx], offs=offs_of(halves).to(DEV))
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+    # linearity in A: f(2a) == 2 f(a) exactly in bf16 (power-of-two scaling)
+    out3 = grouped_mm(ad * 2, bd, offs=offs.to(DEV))
+    assert torch.equal((out * 2).view(torch.int16), out3.view(torch.int16))
+    # against the generic family on a band that crosses a group boundary
+    with K_.forced_path("generic"):
+        ref_band = grouped_mm(ad[4700:4900], bd[:2], offs=torch.tensor([112, 200], dtype=torch.int32, device=DEV))
+    oracle.assert_close(out[4700:4900].cpu(), ref_band.cpu(), 4096)
+
+
+def test_fine_grained_moe_full_size(golden_dir):
+    sizes = _sizes(golden_dir, "fine_grained_top8_g128")
+    offs = offs_of(sizes)
+    a = rnd(torch.Generator().manual_seed(1), 32768, 2048)
+    b = rnd(torch.Generator().manual_seed(2), 128, 2048, 768, scale=0.02)
+    out = torch.full((32768, 768), float("nan"), device=DEV, dtype=torch.bfloat16)
+    K_.grouped_mm_2d3d(a.to(DEV), b.to(DEV), offs.to(DEV), out)
+    assert K_.last_path() == "mfma"
+    want = oracle.grouped_mm(a, b, offs)  # 0.1 TFLOP: a few seconds on the host
+    assert not torch.isnan(out.float()).any()
+    oracle.assert_close(out.cpu(), want, 2048)
+
+
+@pytest.mark.parametrize("b_col", [False, True])
+def test_batched_3d3d_full_size(b_col):
+    a = rnd(torch.Generator().manual_seed(1), 32, 1024, 1024)
+    b = rnd(torch.Generator().manual_seed(2), 32, 1024, 4096, scale=0.02)
+    bd = b.to(DEV)
+    if b_col:
+        bd = bd.transpose(1, 2).contiguous().transpose(1, 2)
+    out = grouped_mm(a.to(DEV), bd)
+    assert K_.last_path() == "mfma"
+    for g in (0, 13, 31):
+        want = (a[g].float() @ b[g].float()).to(torch.bfloat16)
+        oracle.assert_close(out[g].cpu(), want, 1024, what=f"batch {g}")
+
+
+def test_k_grouped_weight_gradient_full_size(golden_dir):
+    sizes = _sizes(golden_dir, "mixtral_top2_g8")
+    offs = offs_of(sizes)
+    a = rnd(torch.Generator().manual_seed(1), 4096, 16384)
+    b = rnd(torch.Generator().manual_seed(2), 16384, 14336)
+    ad, bd = a.to(DEV), b.to(DEV)
+    out = torch.full((8, 4096, 14336), float("nan"), device=DEV, dtype=torch.float32)
+    K_.grouped_mm_2d2d(ad, bd, offs.to(DEV), out)
+    assert K_.last_path() == "mfma"
+    assert not torch.isnan(out).any()
+    rngs = oracle.group_ranges(offs.tolist())
+    for g in (0, 3, 7):
+        s, e = rngs[g]
+        rows = [0, 255, 256, 4095]
+        want = a[rows][:, s:e].float() @ b[s:e].float()
+        torch.testing.assert_close(out[g][rows].cpu(), want, rtol=1.6e-2, atol=1e-2 * ((e - s) / 64) ** 0.5)
+    # the groups partition K: their sum is the plain product (checked on a row band)
+    total = out[:, :64].sum(0).cpu()
+    torch.testing.assert_close(total, a[:64].float() @ b.float(), rtol=1.6e-2, atol=0.5)

@@ -1,0 +1,133 @@
+"""The tile scheduler (csrc/gmm_sched.h), run on the host exactly as the kernels
+run it on the device: every element a group owns is covered by exactly one tile
+of that group, nothing else is covered, and the XCD renumbering is a permutation."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from grouped_mm_bf16_amd import _lib
+
+NONE, ROWS, COLS, CONTRACTION = 0, 1, 2, 3
+
+
+def tile_list(sizes, jag, M, N, K, bm, bn, align=1, remap=0, num_wg=256):
+    lib = _lib.load()
+    offs = np.cumsum(sizes).astype(np.int32) if jag != NONE else np.zeros(1, np.int32)
+    G = len(sizes)
+    n = lib.gmm_host_tile_list(offs.ctypes.data, G, jag, M, N, K, bm, bn, align, remap, num_wg, None, 0)
+    assert n >= 0
+    rec = np.zeros((max(n, 1), 9), np.int32)
+    n2 = lib.gmm_host_tile_list(offs.ctypes.data, G, jag, M, N, K, bm, bn, align, remap, num_wg, rec.ctypes.data, n)
+    assert n2 == n
+    return rec[:n]
+
+
+def coverage(rec, G, M, N, bm, bn, per_group_out):
+    """count[g or 0, m, n] = number of tiles that store element (m, n)."""
+    cnt = np.zeros((G if per_group_out else 1, M, N), np.int32)
+    for g, m0, n0, m_lo, m_hi, n_lo, n_hi, _, _ in rec:
+        r0, r1 = max(m0, m_lo), min(m0 + bm, m_hi)
+        c0, c1 = max(n0, n_lo), min(n0 + bn, n_hi)
+        if r1 > r0 and c1 > c0:
+            cnt[g if per_group_out else 0, r0:r1, c0:c1] += 1
+    return cnt
+
+
+SIZE_LISTS = [
+    [0, 7, 1, 13, 0, 11], [32, 32, 32], [10, 10, 10, 2], [31, 1, 31], [40, 30, 10, 7],
+    [32, 16, 0, 0, 0], [1, 0] * 6, [5, 0, 7, 0, 3, 9], [300, 0, 1, 255, 256, 257, 33], [0, 0, 0],
+]
+
+
+@pytest.mark.parametrize("sizes", SIZE_LISTS)
+@pytest.mark.parametrize("bm,align", [(32, 1), (256, 1), (32, 8), (256, 8), (16, 8)])
+def test_jagged_rows_exact_cover(sizes, bm, align):
+    M, N = sum(sizes), 70
+    if M == 0:
+        assert len(tile_list(sizes, ROWS, 0, N, 16, bm, 64, align)) == 0
+        return
+    rec = tile_list(sizes, ROWS, M, N, 16, bm, 64, align)
+    cnt = coverage(rec, len(sizes), M, N, bm, 64, False)
+    assert (cnt == 1).all()
+    offs = np.cumsum(sizes)
+    for g, m0, n0, m_lo, m_hi, *_ in rec:
+        assert sizes[g] > 0 and m_hi == offs[g] and m_lo == offs[g] - sizes[g]
+        assert m0 % align == 0 and m0 + bm > m_lo and m0 < m_hi  # no tile is pure waste
+        assert n0 % 64 == 0
+
+
+@pytest.mark.parametrize("sizes", SIZE_LISTS)
+@pytest.mark.parametrize("bn,align", [(64, 1), (256, 8)])
+def test_jagged_columns_exact_cover(sizes, bn, align):
+    M, N = 50, sum(sizes)
+    if N == 0:
+        return
+    rec = tile_list(sizes, COLS, M, N, 16, 32, bn, align)
+    assert (coverage(rec, len(sizes), M, N, 32, bn, False) == 1).all()
+    assert all(sizes[r[0]] > 0 for r in rec)
+
+
+@pytest.mark.parametrize("sizes", SIZE_LISTS)
+def test_jagged_contraction_covers_every_group_including_empty(sizes):
+    M, N, K = 70, 90, sum(sizes)
+    rec = tile_list(sizes, CONTRACTION, M, N, K, 64, 64)
+    cnt = coverage(rec, len(sizes), M, N, 64, 64, True)
+    assert (cnt == 1).all()  # also the empty groups: they must be zero-filled
+    offs = np.cumsum(sizes)
+    for r in rec:
+        assert r[7] == offs[r[0]] - sizes[r[0]] and r[8] == offs[r[0]]
+
+
+def test_batched_grid():
+    rec = tile_list([0] * 5, NONE, 100, 130, 16, 64, 64)
+    assert len(rec) == 5 * 2 * 3
+    assert (coverage(rec, 5, 100, 130, 64, 64, True) == 1).all()
+
+
+def test_1023_groups_alternating():
+    sizes = [1 if i % 2 == 0 else 0 for i in range(1023)]
+    sizes[-1] = 0
+    M = sum(sizes)
+    rec = tile_list(sizes, ROWS, M, 8, 8, 256, 256)
+    assert len(rec) == M and (coverage(rec, 1023, M, 8, 256, 256, False) == 1).all()
+    assert sorted(r[0] for r in rec) == [g for g in range(1023) if sizes[g]]
+
+
+@pytest.mark.parametrize("total_like", [[5000], [256 * 3], [1], [255, 300, 7, 1000]])
+def test_xcd_renumbering_is_a_permutation(total_like):
+    sizes = total_like
+    plain = tile_list(sizes, ROWS, sum(sizes), 512, 16, 16, 64, 1, remap=0)
+    remap = tile_list(sizes, ROWS, sum(sizes), 512, 16, 16, 64, 1, remap=1, num_wg=256)
+    assert len(plain) == len(remap)
+    key = lambda r: tuple(r)
+    assert sorted(map(key, plain)) == sorted(map(key, remap))
+    # workgroups of one XCD (ids equal mod 8) get consecutive tiles of the plain order
+    order = {key(r): i for i, r in enumerate(plain)}
+    span = remap[:256]
+    for x in range(8):
+        ids = [order[key(r)] for r in span[x::8]]
+        assert ids == list(range(ids[0], ids[0] + len(ids)))
+
+
+def test_malformed_offsets_never_leave_the_tensor():
+    lib = _lib.load()
+    offs = np.array([5, 3, 100, -4, 20], np.int32)  # decreasing, too large, negative
+    rec = np.zeros((64, 9), np.int32)
+    n = lib.gmm_host_tile_list(offs.ctypes.data, 5, ROWS, 20, 8, 8, 16, 16, 1, 0, 8, rec.ctypes.data, 64)
+    assert 0 <= n <= 64
+    for g, m0, n0, m_lo, m_hi, *_ in rec[:n]:
+        assert 0 <= m_lo <= m_hi <= 20 and 0 <= m0 < 20
+
+
+def test_random_lists_exact_cover():
+    rng = np.random.default_rng(1)
+    for _ in range(60):
+        G = int(rng.integers(1, 30))
+        sizes = (rng.integers(0, 80, size=G) * (rng.random(G) > 0.3)).astype(int).tolist()
+        if sum(sizes) == 0:
+            continue
+        bm = int(rng.choice([16, 32, 64, 256]))
+        align = int(rng.choice([1, 8]))
+        rec = tile_list(sizes, ROWS, sum(sizes), 40, 8, bm, 32, align, remap=int(rng.integers(0, 2)), num_wg=16)
+        assert (coverage(rec, G, sum(sizes), 40, bm, 32, False) == 1).all()
