@@ -1,0 +1,390 @@
+#!/usr/bin/env python3
+"""Generates gmm_tile_asm.inc: the per-tile main loop and epilogue of the MFMA
+grouped GEMM kernels as hand-scheduled gfx950 assembly.
+
+    python gen_tile_asm.py > gmm_tile_asm.inc      (build.py does this)
+
+Why generated assembly: the loop keeps 256 accumulator registers, two sets of
+MFMA operand fragments and sixteen in-flight direct-to-LDS copies alive at once.
+Written as C++ the compiler spills inside the loop, and every spill reload waits
+on the vector-memory counter that the asynchronous copies also use, which stalls
+the pipeline.  Here every register is named, so nothing is spilled and the issue
+order is exactly the one below.
+
+One block computes one 256 x 256 output tile with 4 waves (2 x 2, 128 x 128 per
+wave, 4 x 4 MFMA blocks of 32 x 32):
+
+  * K is walked in tiles of 64; A and B tiles are copied global -> LDS by
+    buffer_load_dwordx4 ... lds (no registers involved) into two buffers;
+  * an operand that is contiguous along K lives in LDS as [row][64 k] with its
+    16-byte chunks XOR-swizzled (conflict-free ds_read_b128 fragments); one that
+    is contiguous along M / N lives as [k][256] in blocks of two k rows with a
+    64-byte pad, read with ds_read_b64_tr_b16 (the LDS transposes 4 x 16 blocks);
+  * per k16 step a wave issues 16 v_mfma_f32_32x32x16_bf16 and, between them, the
+    8 fragment reads of the next step and its share of the copies of the next
+    tiles, so the matrix pipe never waits on LDS latency;
+  * one s_barrier per K tile, placed after step 2 so that step 3's MFMAs run
+    while the barrier's stragglers arrive and the first fragments of the next
+    tile are fetched under them;
+  * epilogue, bf16: the MFMA operands are swapped so a lane owns 4 consecutive
+    columns, packs them (v_cvt_pk_bf16_f32), stages the wave's 128 x 128 block in
+    LDS and writes 16 bytes per lane, 256 contiguous bytes per row;
+    fp32: each accumulator register goes out as one dword store, 128 contiguous
+    bytes per row.
+
+Registers (fixed):
+  a[0:255]     accumulators, block (i, j) at a[(4 i + j) 16 ...]
+  v[0:15]      A fragments set 0, v[16:31] set 1, v[32:47] B set 0, v[48:63] B set 1
+  v[64:95]     temporaries
+  inputs are pinned by the C++ wrapper to v[128:...] and s[36:...] (see TileRegs).
+"""
+import sys
+
+PITCH = 272           # bytes per staged row of 128 bf16 (256 + 16: shifts banks per row)
+TR_BLOCK = 1088       # two k rows of 512 bytes + 64 bytes pad
+KC_STAGE = 256 * 64 * 2
+TR_STAGE = 32 * TR_BLOCK
+STAGE_BYTES = 4 * 128 * PITCH
+
+# ---- fixed register map ----------------------------------------------------
+V_AF = [0, 16]        # A fragment sets (4 x 4 registers each)
+V_BF = [32, 48]
+V_TMP = 64            # 64..95
+V_VOA_HEAD, V_VOB_HEAD = 128, 136
+V_VOA, V_VOB = 144, 152
+V_VOA_TAIL, V_VOB_TAIL = 160, 168
+V_RA, V_RB = 176, 180  # fragment read addresses (4 + 4)
+V_EPI = 184            # 184: stage write addr, 185: stage read addr, 186: store voffset, 187: row - row_lo
+V_OOB = 188            # constant 0x80000000
+
+S_RA, S_RB, S_RC = 36, 40, 44   # buffer resources
+S_SC = 48                        # scalars s[48:55]
+S_NK, S_ASTEP, S_BSTEP, S_LDS, S_ROWCNT, S_CSTEP, S_NVALID, S_SPARE = range(48, 56)
+S_T = 56                         # temporaries s[56:79]
+
+
+class Emit:
+    def __init__(self):
+        self.lines = []
+
+    def __call__(self, s):
+        self.lines.append(s)
+
+    def label(self, name):
+        self.lines.append(name + ":")
+
+    def text(self):
+        return "\n".join('      "%s\\n\\t"' % l for l in self.lines)
+
+
+def acc(i, j):
+    return (4 * i + j) * 16
+
+
+def vr(base, n=1):
+    return "v%d" % base if n == 1 else "v[%d:%d]" % (base, base + n - 1)
+
+
+def sr(base, n=1):
+    return "s%d" % base if n == 1 else "s[%d:%d]" % (base, base + n - 1)
+
+
+class Variant:
+    def __init__(self, a_tr, b_tr, out_f32):
+        self.a_tr, self.b_tr, self.out_f32 = a_tr, b_tr, out_f32
+        self.a_stage = TR_STAGE if a_tr else KC_STAGE
+        self.b_stage = TR_STAGE if b_tr else KC_STAGE
+        self.b_base = 2 * self.a_stage          # LDS offset of B buffer 0
+        self.swap = not out_f32                  # bf16: lanes own 4 consecutive columns
+        self.name = "%s%s_%s" % ("t" if a_tr else "k", "t" if b_tr else "k", "f32" if out_f32 else "bf16")
+
+    # -- fragment reads of k16 step `s` of buffer `buf` into register set `st`; returns list of instr
+    def frag_reads(self, buf, s, st):
+        out = []
+        for op, tr, vbase, vaddr, stage, lbase in (
+            ("A", self.a_tr, V_AF[st], V_RA, self.a_stage, 0),
+            ("B", self.b_tr, V_BF[st], V_RB, self.b_stage, 0),
+        ):
+            for x in range(4):
+                d = vbase + 4 * x
+                if not tr:
+                    # address register per step; sub-tiles are 32 rows = 4096 bytes apart
+                    out.append("ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(vaddr + s), buf * stage + x * 4096))
+                else:
+                    o = buf * stage + s * 8 * TR_BLOCK + x * 64
+                    out.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d, 2), vr(vaddr), o))
+                    out.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d + 2, 2), vr(vaddr), o + 512))
+        return out
+
+    def n_frag_reads(self):
+        return 4 * (2 if self.a_tr else 1) + 4 * (2 if self.b_tr else 1)
+
+    # -- MFMAs of one step on register set st
+    def mfmas(self, st):
+        out = []
+        for i in range(4):
+            for j in range(4):
+                a = vr(V_AF[st] + 4 * i, 4)
+                b = vr(V_BF[st] + 4 * j, 4)
+                c = "a[%d:%d]" % (acc(i, j), acc(i, j) + 15)
+                x, y = (b, a) if self.swap else (a, b)
+                out.append("v_mfma_f32_32x32x16_bf16 %s, %s, %s, %s" % (c, x, y, c))
+        return out
+
+    # -- copy instruction n (0..15) of a K tile into buffer buf.
+    # s_tail / s_oob: SGPR pairs (lane masks all-ones / zero): use the tail offsets / kill the copy.
+    # s_ka / s_kb: SGPRs with the tile's byte offsets along K for A and B.  which: "head" or "loop".
+    def dma(self, n, buf, which, s_tail, s_oob, s_ka, s_kb, tmp):
+        out = []
+        is_a = n < 8
+        i = n if is_a else n - 8
+        tr = self.a_tr if is_a else self.b_tr
+        stage = self.a_stage if is_a else self.b_stage
+        lbase = 0 if is_a else self.b_base
+        # per wave: 8 instructions of 1 KiB each; wave w covers [w * 8 KiB, (w + 1) * 8 KiB) of the
+        # stage (row-chunk layout) or blocks w * 8 .. w * 8 + 7 (transposed layout): the wave part of
+        # the LDS address is in s[S_T + 20] (A) / s[S_T + 21] (B), set up by the prologue.
+        blk = TR_BLOCK if tr else 1024
+        lds_off = lbase + buf * stage + i * blk
+        s_wave = S_T + 20 + (0 if is_a else 1)
+        if which == "head":
+            vo = (V_VOA_HEAD if is_a else V_VOB_HEAD) + i
+            src = vr(vo)
+        else:
+            vn = (V_VOA if is_a else V_VOB) + i
+            vt = (V_VOA_TAIL if is_a else V_VOB_TAIL) + i
+            out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(vn), vr(vt), sr(s_tail, 2)))
+            out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(tmp), vr(V_OOB), sr(s_oob, 2)))
+            src = vr(tmp)
+        out.append("s_add_u32 m0, %s, %d" % (sr(s_wave), lds_off))
+        out.append("s_nop 0")
+        out.append("buffer_load_dwordx4 %s, %s, %s offen lds" % (src, sr(S_RA if is_a else S_RB, 4), sr(s_ka if is_a else s_kb)))
+        return out
+
+
+def interleave(e, mfmas, side_groups):
+    """Emit 16 MFMAs with the side groups spread between them (one group after each MFMA, in order)."""
+    n = len(mfmas)
+    slots = [[] for _ in range(n)]
+    # spread groups evenly over the first n - 1 gaps
+    g = len(side_groups)
+    for k, grp in enumerate(side_groups):
+        slots[min(n - 1, (k * n) // max(g, 1))].extend(grp)
+    for k in range(n):
+        e(mfmas[k])
+        for ins in slots[k]:
+            e(ins)
+
+
+def gen_variant(v):
+    e = Emit()
+    L = "%s_%%=" % v.name  # unique label suffix per asm instance
+    sT = S_T
+    # temporaries
+    s_kt, s_t1 = sT + 0, sT + 1
+    s_ka1, s_kb1 = sT + 2, sT + 3       # K offsets of tile kt + 1
+    s_ka2, s_kb2 = sT + 4, sT + 5       # K offsets of tile kt + 2
+    s_tail1, s_oob1 = sT + 6, sT + 8    # pairs
+    s_tail2, s_oob2 = sT + 10, sT + 12
+    s_last = sT + 14                    # nk - 1
+    s_zero = sT + 15
+    s_waveA, s_waveB = sT + 20, sT + 21
+
+    def tile_masks(s_tile, s_tail, s_oob):
+        # tail mask: tile == nk - 1 ; oob mask: tile >= nk
+        e("s_cmp_eq_u32 %s, %s" % (sr(s_tile), sr(s_last)))
+        e("s_cselect_b64 %s, -1, 0" % sr(s_tail, 2))
+        e("s_cmp_ge_u32 %s, %s" % (sr(s_tile), sr(S_NK)))
+        e("s_cselect_b64 %s, -1, 0" % sr(s_oob, 2))
+
+    # ------------------------------------------------------------------ prologue
+    e("; ---- prologue (%s)" % v.name)
+    e("v_mov_b32 %s, 0x80000000" % vr(V_OOB))
+    e("s_sub_u32 %s, %s, 1" % (sr(s_last), sr(S_NK)))
+    e("s_mov_b32 %s, 0" % sr(s_zero))
+    # wave part of the LDS copy destinations: wave id is in s[S_SPARE]
+    e("s_mul_i32 %s, %s, %d" % (sr(s_waveA), sr(S_SPARE), 8 * (TR_BLOCK if v.a_tr else 1024)))
+    e("s_add_u32 %s, %s, %s" % (sr(s_waveA), sr(s_waveA), sr(S_LDS)))
+    e("s_mul_i32 %s, %s, %d" % (sr(s_waveB), sr(S_SPARE), 8 * (TR_BLOCK if v.b_tr else 1024)))
+    e("s_add_u32 %s, %s, %s" % (sr(s_waveB), sr(s_waveB), sr(S_LDS)))
+    # tile 0 -> buffer 0 (head offsets)
+    for n in range(16):
+        for ins in v.dma(n, 0, "head", 0, 0, s_zero, s_zero, V_TMP):
+            e(ins)
+    # tile 1 -> buffer 1, first 6 copies
+    e("s_mov_b32 %s, 1" % sr(s_t1))
+    tile_masks(s_t1, s_tail1, s_oob1)
+    e("s_mov_b32 %s, %s" % (sr(s_ka1), sr(S_ASTEP)))
+    e("s_mov_b32 %s, %s" % (sr(s_kb1), sr(S_BSTEP)))
+    for n in range(6):
+        for ins in v.dma(n, 1, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + n):
+            e(ins)
+    # zero the accumulators while the copies fly
+    for r in range(256):
+        e("v_accvgpr_write_b32 a%d, 0" % r)
+    e("s_waitcnt vmcnt(6)")
+    e("s_barrier")
+    for ins in v.frag_reads(0, 0, 0):
+        e(ins)
+    e("s_mov_b32 %s, 0" % sr(s_kt))
+    e("s_cmp_eq_u32 %s, 0" % sr(S_NK))
+    e("s_cbranch_scc1 L_done_%s" % L)
+
+    # ------------------------------------------------------------------ K loop, two tiles per trip
+    def ktile(buf):
+        # on entry: fragments of step 0 in set 0 (in flight); copies 0..5 of tile kt+1 in flight
+        e("; ---- k tile on buffer %d" % buf)
+        # K offsets and masks of tiles kt+1 and kt+2
+        e("s_add_u32 %s, %s, 1" % (sr(s_t1), sr(s_kt)))
+        tile_masks(s_t1, s_tail1, s_oob1)
+        e("s_mul_i32 %s, %s, %s" % (sr(s_ka1), sr(s_t1), sr(S_ASTEP)))
+        e("s_mul_i32 %s, %s, %s" % (sr(s_kb1), sr(s_t1), sr(S_BSTEP)))
+        e("s_add_u32 %s, %s, 2" % (sr(s_t1), sr(s_kt)))
+        tile_masks(s_t1, s_tail2, s_oob2)
+        e("s_mul_i32 %s, %s, %s" % (sr(s_ka2), sr(s_t1), sr(S_ASTEP)))
+        e("s_mul_i32 %s, %s, %s" % (sr(s_kb2), sr(s_t1), sr(S_BSTEP)))
+        nb = buf ^ 1
+        # step 0: MFMA set 0, read step 1 -> set 1, copies 6..10 of tile kt+1 -> other buffer
+        e("s_waitcnt lgkmcnt(0)")
+        side = [[x] for x in v.frag_reads(buf, 1, 1)]
+        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(6, 11)]
+        interleave(e, v.mfmas(0), side)
+        # step 1
+        e("s_waitcnt lgkmcnt(0)")
+        side = [[x] for x in v.frag_reads(buf, 2, 0)]
+        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(11, 16)]
+        interleave(e, v.mfmas(1), side)
+        # step 2
+        e("s_waitcnt lgkmcnt(0)")
+        side = [[x] for x in v.frag_reads(buf, 3, 1)]
+        interleave(e, v.mfmas(0), side)
+        # tile kt+1 has landed for this wave; after the barrier for all, and `buf` is free
+        e("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        e("s_barrier")
+        # step 3: MFMA set 1, read step 0 of the next tile -> set 0, copies 0..5 of tile kt+2 -> buf
+        side = [[x] for x in v.frag_reads(nb, 0, 0)]
+        side += [v.dma(n, buf, "loop", s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, 6)]
+        interleave(e, v.mfmas(1), side)
+        e("s_add_u32 %s, %s, 1" % (sr(s_kt), sr(s_kt)))
+
+    e.label("L_loop_%s" % L)
+    ktile(0)
+    e("s_cmp_ge_u32 %s, %s" % (sr(s_kt), sr(S_NK)))
+    e("s_cbranch_scc1 L_done_%s" % L)
+    ktile(1)
+    e("s_cmp_lt_u32 %s, %s" % (sr(s_kt), sr(S_NK)))
+    e("s_cbranch_scc1 L_loop_%s" % L)
+    e.label("L_done_%s" % L)
+
+    # ------------------------------------------------------------------ epilogue
+    e("; ---- epilogue")
+    e("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    e("s_nop 15")
+    e("s_nop 15")
+    e("s_barrier")
+    if not v.out_f32:
+        # acc block (i, j), register 4 q + r  ->  C[m = 32 i + lane % 32][n = 32 j + 8 q + 4 (lane / 32) + r]
+        t = V_TMP
+        k = 0
+        for i in range(4):
+            for j in range(4):
+                for q in range(4):
+                    b = t + 6 * (k % 4)
+                    k += 1
+                    a0 = acc(i, j) + 4 * q
+                    for r in range(4):
+                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), a0 + r))
+                    e("v_cvt_pk_bf16_f32 %s, %s, %s" % (vr(b + 4), vr(b), vr(b + 1)))
+                    e("v_cvt_pk_bf16_f32 %s, %s, %s" % (vr(b + 5), vr(b + 2), vr(b + 3)))
+                    e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 4, 2), (32 * i) * PITCH + (32 * j + 8 * q) * 2))
+        e("s_waitcnt lgkmcnt(0)")
+        # read back: instruction r covers rows 4 r .. 4 r + 3 (16 lanes of 16 bytes per row)
+        # v[V_EPI + 2] = store offset of row 0 (or OOB when the lane's columns are invalid)
+        # v[V_EPI + 3] = (row of this lane at r = 0) - row_lo ; valid iff (unsigned)(that + 4 r) < S_ROWCNT
+        depth = 4
+        regs = [t + 4 * x for x in range(depth)]          # data, 4 regs each (64..79)
+        voff, vrow, vsel = t + 16, t + 17, t + 18
+        e("v_mov_b32 %s, %s" % (vr(voff), vr(V_EPI + 2)))
+        e("v_mov_b32 %s, %s" % (vr(vrow), vr(V_EPI + 3)))
+        for r in range(depth):
+            e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r], 4), vr(V_EPI + 1), r * 4 * PITCH))
+        for r in range(32):
+            e("s_waitcnt lgkmcnt(%d)" % min(depth - 1, 31 - r))
+            e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
+            e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vsel), vr(V_OOB), vr(voff)))
+            e("buffer_store_dwordx4 %s, %s, %s, 0 offen" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
+            if r + depth < 32:
+                # the store above must have read its data before the register is reloaded
+                e("s_nop 0")
+                e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r % depth], 4), vr(V_EPI + 1), (r + depth) * 4 * PITCH))
+            e("v_add_u32 %s, %s, %s" % (vr(voff), sr(S_CSTEP), vr(voff)))
+            e("v_add_u32 %s, 4, %s" % (vr(vrow), vr(vrow)))
+    else:
+        # acc block (i, j), register 4 q + r -> C[m = 32 i + 8 q + 4 (lane / 32) + r][n = 32 j + lane % 32]
+        # v[V_EPI + 2] = store offset of (row 4 (lane / 32), col lane % 32); v[V_EPI + 3] = 4 (lane / 32) - row_lo
+        # column validity of block j: lane mask pairs s[S_T + 24 + 2 j]
+        t = V_TMP
+        voff, vrow, vsel = t + 16, t + 17, t + 18
+        for j in range(4):
+            e("v_add_u32 %s, %d, %s" % (vr(t + 19), 32 * j, vr(V_EPI + 1)))   # V_EPI + 1 = lane % 32 (column in block)
+            e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_NVALID), vr(t + 19)))
+            e("s_mov_b64 %s, vcc" % sr(S_T + 24 + 2 * j, 2))
+        k = 0
+        e("s_mov_b32 %s, 0" % sr(S_T + 16))   # running row offset in bytes
+        for i in range(4):
+            for q in range(4):
+                for r in range(4):
+                    row = 32 * i + 8 * q + r
+                    e("v_add_u32 %s, %d, %s" % (vr(vrow), row, vr(V_EPI + 3)))
+                    e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
+                    e("s_mov_b64 %s, vcc" % sr(S_T + 32, 2))
+                    e("s_mul_i32 %s, %s, %d" % (sr(S_T + 16), sr(S_CSTEP), row))
+                    for j in range(4):
+                        b = t + (k % 8)
+                        k += 1
+                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b), acc(i, j) + 4 * q + r))
+                        e("s_and_b64 vcc, %s, %s" % (sr(S_T + 32, 2), sr(S_T + 24 + 2 * j, 2)))
+                        e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(t + 8 + (k % 8)), vr(V_OOB), vr(V_EPI + 2)))
+                        e("buffer_store_dword %s, %s, %s, %s offen offset:%d" % (vr(b), vr(t + 8 + (k % 8)), sr(S_RC, 4), sr(S_T + 16), 128 * j))
+    e("s_waitcnt lgkmcnt(0)")
+    e("s_barrier")
+    return e
+
+
+def clobbers():
+    c = ["memory", "vcc", "scc"]
+    c += ["v%d" % i for i in range(0, 96)] + ["v%d" % V_OOB]
+    c += ["a%d" % i for i in range(256)]
+    c += ["s%d" % i for i in range(S_T, S_T + 34)]
+    return ", ".join('"%s"' % x for x in c)
+
+
+def main():
+    out = []
+    out.append("// Generated by gen_tile_asm.py -- do not edit.")
+    out.append("// Per-tile main loop + epilogue in gfx950 assembly, one function per operand-layout / output variant.")
+    out.append("#define GMM_TILE_PITCH %d" % PITCH)
+    out.append("#define GMM_TILE_TR_BLOCK %d" % TR_BLOCK)
+    out.append("#define GMM_TILE_KC_STAGE %d" % KC_STAGE)
+    out.append("#define GMM_TILE_TR_STAGE %d" % TR_STAGE)
+    out.append("#define GMM_TILE_STAGING_BYTES %d" % STAGE_BYTES)
+    for a_tr in (0, 1):
+        for b_tr in (0, 1):
+            for f32 in (0, 1):
+                v = Variant(a_tr, b_tr, f32)
+                e = gen_variant(v)
+                out.append("")
+                out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d>(const GmmTileRegs& r) {" % (a_tr, b_tr, f32))
+                out.append("  asm volatile(")
+                out.append(e.text())
+                out.append("      :")
+                out.append('      : "{v[128:135]}"(r.voa_head), "{v[136:143]}"(r.vob_head), "{v[144:151]}"(r.voa), "{v[152:159]}"(r.vob),')
+                out.append('        "{v[160:167]}"(r.voa_tail), "{v[168:175]}"(r.vob_tail), "{v[176:179]}"(r.ra_addr), "{v[180:183]}"(r.rb_addr),')
+                out.append('        "{v[184:187]}"(r.epi), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
+                out.append("      : %s);" % clobbers())
+                out.append("}")
+    sys.stdout.write("\n".join(out) + "\n")
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,140 @@
+// One 256 x 256 output tile of C = A * B on gfx950: C++ wrapper around the generated assembly
+// (gmm_tile_asm.inc, made by gen_tile_asm.py).  The wrapper turns a tile description into the
+// per-lane offsets and the scalars the assembly expects in fixed registers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int gmm_v4i __attribute__((ext_vector_type(4)));
+typedef int gmm_v8i __attribute__((ext_vector_type(8)));
+
+struct GmmTileRegs {
+  gmm_v8i voa_head, vob_head;  // copy offsets of K tile 0 (first/last chunk masks applied)
+  gmm_v8i voa, vob;            // copy offsets of a full K tile
+  gmm_v8i voa_tail, vob_tail;  // copy offsets of the last K tile
+  gmm_v4i ra_addr, rb_addr;    // LDS fragment read addresses
+  gmm_v4i epi;                 // epilogue: per-lane addresses (see gen_tile_asm.py)
+  gmm_v4i rsrc_a, rsrc_b, rsrc_c;
+  gmm_v8i scal;                // nk, a_step, b_step, lds_base, row_cnt, c_step, n_valid, wave
+};
+
+template <int A_TR, int B_TR, int OUT_F32>
+__device__ __forceinline__ void gmm_tile_asm(const GmmTileRegs& r);
+
+#include "gmm_tile_asm.inc"
+
+constexpr int GMM_TILE_M = 256, GMM_TILE_N = 256, GMM_TILE_K = 64;
+constexpr unsigned GMM_OOB = 0x80000000u;
+
+// LDS bytes one workgroup needs for a layout pair (pipeline buffers or the bf16 staging area).
+template <int A_TR, int B_TR>
+constexpr int gmm_tile_lds_bytes() {
+  constexpr int pipe = 2 * (A_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE) + 2 * (B_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE);
+  return pipe > GMM_TILE_STAGING_BYTES ? pipe : GMM_TILE_STAGING_BYTES;
+}
+
+__device__ __forceinline__ gmm_v4i gmm_make_rsrc(const void* p, long long bytes) {
+  const unsigned long long a = (unsigned long long)p;
+  if (bytes < 0) bytes = 0;
+  if (bytes > 0x7fffffffLL) bytes = 0x7fffffffLL;
+  gmm_v4i r = {(int)(unsigned)a, (int)(unsigned)((a >> 32) & 0xffffu), (int)bytes, 0x00020000};
+  return r;
+}
+
+__device__ __forceinline__ int gmm_swz(int row) { return (row >> 1) & 7; }
+
+// One operand of a tile.  `base` points at element (row 0 of the tile, k_begin) of the operand;
+// `ld` is the leading dimension in elements; `bytes` is the distance from `base` to the end of the
+// operand's storage (reads past it return zero).
+struct GmmOperand {
+  const uint16_t* base;
+  int ld;
+  long long bytes;
+};
+
+// Description of one tile for the assembly.  klen = number of k elements from k_begin that count.
+struct GmmTileDesc {
+  GmmOperand a, b;
+  void* c;               // element (m0, n0) of the output
+  int ldc;
+  long long c_bytes;     // from c to the end of the output storage
+  int klen;
+  int row_rel0;          // m0 - m_lo   (may be negative: rows before m_lo are not stored)
+  int row_cnt;           // m_hi - m_lo
+  int col_lo, col_hi;    // columns [col_lo, col_hi) of the tile are stored (relative to n0)
+};
+
+template <int TR>
+__device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int klen, int nk,
+                                                 gmm_v8i& head, gmm_v8i& full, gmm_v8i& tail) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    int k, vo;
+    if (!TR) {
+      const int row = wave * 64 + i * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ gmm_swz(row);
+      k = c * 8;
+      vo = row * ld * 2 + c * 16;
+    } else {
+      const int blk = wave * 8 + i;
+      k = 8 * (blk >> 2) + (blk & 3) + 4 * (lane >> 5);
+      vo = k * ld * 2 + (lane & 31) * 16;
+    }
+    full[i] = vo;
+    head[i] = (k < klen) ? vo : (int)GMM_OOB;
+    tail[i] = ((nk - 1) * GMM_TILE_K + k < klen) ? vo : (int)GMM_OOB;
+  }
+}
+
+template <int A_TR, int B_TR, int OUT_F32>
+__device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave) {
+  constexpr int A_STAGE = A_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int nk = (t.klen + GMM_TILE_K - 1) / GMM_TILE_K;
+  GmmTileRegs r;
+  gmm_copy_offsets<A_TR>(lane, wave, t.a.ld, t.klen, nk, r.voa_head, r.voa, r.voa_tail);
+  gmm_copy_offsets<B_TR>(lane, wave, t.b.ld, t.klen, nk, r.vob_head, r.vob, r.vob_tail);
+  const int q = lane >> 4, ii = lane & 15;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int chunk = 2 * s + (lane >> 5);
+    if (!A_TR) {
+      const int row = wm * 128 + (lane & 31);
+      r.ra_addr[s] = lds_base + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
+    } else {
+      r.ra_addr[s] = lds_base + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wm * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
+    }
+    if (!B_TR) {
+      const int row = wn * 128 + (lane & 31);
+      r.rb_addr[s] = lds_base + 2 * A_STAGE + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
+    } else {
+      r.rb_addr[s] = lds_base + 2 * A_STAGE + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wn * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
+    }
+  }
+  int c_step, n_valid = 0;
+  if (!OUT_F32) {
+    const int row_t = wm * 128 + (lane >> 4), col_t = wn * 128 + (lane & 15) * 8;
+    r.epi[0] = lds_base + wave * (128 * GMM_TILE_PITCH) + (lane & 31) * GMM_TILE_PITCH + 8 * (lane >> 5);
+    r.epi[1] = lds_base + wave * (128 * GMM_TILE_PITCH) + (lane >> 4) * GMM_TILE_PITCH + (lane & 15) * 16;
+    r.epi[2] = (col_t >= t.col_lo && col_t + 8 <= t.col_hi) ? (row_t * t.ldc + col_t) * 2 : (int)GMM_OOB;
+    r.epi[3] = t.row_rel0 + row_t;
+    c_step = 4 * t.ldc * 2;
+  } else {
+    const int row_t = wm * 128 + 4 * (lane >> 5), col_t = wn * 128 + (lane & 31);
+    r.epi[0] = 0;
+    r.epi[1] = lane & 31;
+    r.epi[2] = (row_t * t.ldc + col_t) * 4;
+    r.epi[3] = t.row_rel0 + row_t;
+    c_step = t.ldc * 4;
+    n_valid = t.col_hi - wn * 128;
+    if (n_valid < 0) n_valid = 0;
+  }
+  r.rsrc_a = gmm_make_rsrc(t.a.base, t.a.bytes);
+  r.rsrc_b = gmm_make_rsrc(t.b.base, t.b.bytes);
+  r.rsrc_c = gmm_make_rsrc(t.c, t.c_bytes);
+  const int a_step = A_TR ? GMM_TILE_K * t.a.ld * 2 : GMM_TILE_K * 2;
+  const int b_step = B_TR ? GMM_TILE_K * t.b.ld * 2 : GMM_TILE_K * 2;
+  gmm_v8i sc = {nk, a_step, b_step, (int)lds_base, t.row_cnt, c_step, n_valid, wave};
+  r.scal = sc;
+  gmm_tile_asm<A_TR, B_TR, OUT_F32>(r);
+}
