@@ -39,7 +39,7 @@ def sources() -> list:
 
 
 def _headers() -> list:
-    hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".inc"))]
     hs.append(os.path.join(HERE, "..", "include", "grouped_mm_hip.h"))
     return hs
 
@@ -61,9 +61,23 @@ def _compile(src: str, force: bool) -> str:
     return obj
 
 
+def generate(force: bool = False) -> str:
+    """Run gen_tile_asm.py -> csrc/gmm_tile_asm.inc (the hand-scheduled tile assembly)."""
+    gen = os.path.join(CSRC, "gen_tile_asm.py")
+    inc = os.path.join(CSRC, "gmm_tile_asm.inc")
+    if force or _stale(inc, [gen]):
+        res = subprocess.run([sys.executable, gen], capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"gen_tile_asm.py failed:\n{res.stderr}")
+        with open(inc, "w") as f:
+            f.write(res.stdout)
+    return inc
+
+
 def build(force: bool = False, verbose: bool = False) -> str:
-    """Compile (when stale or forced) and link; returns the library path."""
+    """Generate, compile (when stale or forced) and link; returns the library path."""
     os.makedirs(OBJ_DIR, exist_ok=True)
+    generate(force)
     srcs = sources()
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), srcs))

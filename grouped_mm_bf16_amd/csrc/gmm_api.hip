@@ -62,6 +62,24 @@ bool mfma_eligible(const Problem& pr, GmmLayout& lay, int& align) {
   return true;
 }
 
+// The generated-assembly tile takes a subset of what the register-staged kernel takes.
+bool asm_tile_eligible(const Problem& pr, const GmmLayout& lay) {
+  const GmmParams& p = pr.p;
+  if (p.jag == GMM_JAG_N) return false;                           // jagged columns: element-masked stores
+  if (p.jag == GMM_JAG_K && (lay.a_kc || lay.b_kc)) return false;  // unaligned k ranges need element masks
+  if (p.c_sn != 1) return false;
+  const int64_t lda = lay.a_kc ? p.a_sm : p.a_sk, ldb = lay.b_kc ? p.b_sn : p.b_sk, ldc = p.c_sm;
+  const int64_t ld_max = int64_t(1) << 22;
+  if (lda >= ld_max || ldb >= ld_max || ldc >= ld_max) return false;
+  // a transposed-layout operand is addressed from its first k row: the whole slice must fit 31 bits
+  if (!lay.a_kc && int64_t(p.K) * lda * 2 >= (int64_t(1) << 31)) return false;
+  if (!lay.b_kc && int64_t(p.K) * ldb * 2 >= (int64_t(1) << 31)) return false;
+  if (pr.out_dtype == GMM_DT_BF16) {
+    if (!aligned16(p.c) || !mult8(p.c_sm) || !mult8(p.c_sg) || !mult8(p.N)) return false;
+  }
+  return true;
+}
+
 int run(Problem& pr, hipStream_t stream) {
   GmmParams& p = pr.p;
   if (!p.a || !p.b || !p.c) return GMM_ERR_BAD_ARGUMENT;
@@ -86,8 +104,10 @@ int run(Problem& pr, hipStream_t stream) {
   if (use_mfma) {
     p.align = align;
     p.xcd_remap = g_xcd_remap.load(std::memory_order_relaxed);
+    const bool can_asm = asm_tile_eligible(pr, lay);
     int cfg = g_forced_config.load(std::memory_order_relaxed);
-    if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = GMM_CFG_256x256;
+    if (cfg == GMM_CFG_ASM_256x256 && !can_asm) return GMM_ERR_UNSUPPORTED;
+    if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = can_asm ? GMM_CFG_ASM_256x256 : GMM_CFG_REG_256x256;
     rc = gmm_launch_mfma(p, lay, pr.out_dtype, cfg, cus, stream);
     t_last_path = GMM_PATH_MFMA;
     t_last_config = cfg;

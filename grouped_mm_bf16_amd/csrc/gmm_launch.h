@@ -14,7 +14,10 @@ struct GmmLayout {
 };
 
 // Tile configurations of the MFMA family.
-enum GmmMfmaConfig : int { GMM_CFG_256x256 = 0, GMM_CFG_COUNT };
+// REG: tiles staged through registers, compiler-scheduled (takes every aligned layout and the
+//      jagged-column / unaligned jagged-contraction cases).
+// ASM: generated assembly tile with direct-to-LDS copies (the fast one).
+enum GmmMfmaConfig : int { GMM_CFG_REG_256x256 = 0, GMM_CFG_ASM_256x256 = 1, GMM_CFG_COUNT };
 
 // bf16 inputs only; out_dtype bf16 or fp32.  Returns like gmm_launch_generic.
 int gmm_launch_mfma(GmmParams p, GmmLayout lay, int out_dtype, int config, int num_cus, hipStream_t stream);

@@ -21,6 +21,7 @@
 // multiples of 8 elements.
 #include "gmm_device.h"
 #include "gmm_launch.h"
+#include "gmm_tile.h"
 
 namespace {
 
@@ -255,6 +256,82 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) gmm_mfma_kernel(cons
   }
 }
 
+
+// ---- kernel built on the generated assembly tile (gmm_tile.h) --------------------------------- //
+// Same tile list, but each tile's main loop and epilogue run as one hand-scheduled assembly block:
+// direct global -> LDS copies, no register staging, explicit registers.  A_TR / B_TR: the operand is
+// contiguous along M / N (not along K) and is read from LDS with transposing loads.
+template <int A_TR, int B_TR, int OUT_F32>
+__global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
+  __shared__ __attribute__((aligned(1024))) char lds[gmm_tile_lds_bytes<A_TR, B_TR>()];
+  __shared__ int32_t cum[GMM_MAX_GROUPS + 1];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
+  constexpr int ESZ = OUT_F32 ? 4 : 2;
+
+  const int total = gmm_build_tile_table<256>(p, GMM_TILE_M, GMM_TILE_N, cum);
+  const uint16_t* __restrict__ A = static_cast<const uint16_t*>(p.a);
+  const uint16_t* __restrict__ B = static_cast<const uint16_t*>(p.b);
+  char* __restrict__ C = static_cast<char*>(p.c);
+  const int lda = int(A_TR ? p.a_sk : p.a_sm);
+  const int ldb = int(B_TR ? p.b_sk : p.b_sn);
+  const int ldc = int(p.c_sm);
+
+  for (int t = blockIdx.x; t < total; t += gridDim.x) {
+    const int tt = p.xcd_remap ? gmm_xcd_remap(t, total, gridDim.x) : t;
+    const GmmTile tile = gmm_locate_tile(p, cum, tt, GMM_TILE_M, GMM_TILE_N);
+    const int g = __builtin_amdgcn_readfirstlane(tile.g);
+    const int m0 = __builtin_amdgcn_readfirstlane(tile.m0), n0 = __builtin_amdgcn_readfirstlane(tile.n0);
+    const int k_lo = __builtin_amdgcn_readfirstlane(tile.k_lo), k_hi = __builtin_amdgcn_readfirstlane(tile.k_hi);
+    // the copies move 16-byte chunks along K for an operand that is contiguous along K
+    const int k_begin = (A_TR && B_TR) ? k_lo : (k_lo & ~7);
+    const uint16_t* a = A + int64_t(g) * p.a_sg;
+    const uint16_t* b = B + int64_t(g) * p.b_sg;
+
+    GmmTileDesc d;
+    d.a.ld = lda;
+    d.b.ld = ldb;
+    if (!A_TR) {
+      d.a.base = a + int64_t(m0) * lda + k_begin;
+      d.a.bytes = (int64_t(p.M - m0) * lda - k_begin) * 2;
+    } else {
+      d.a.base = a + int64_t(k_begin) * lda + m0;
+      d.a.bytes = (int64_t(p.K - k_begin) * lda - m0) * 2;
+    }
+    if (!B_TR) {
+      d.b.base = b + int64_t(n0) * ldb + k_begin;
+      d.b.bytes = (int64_t(p.N - n0) * ldb - k_begin) * 2;
+    } else {
+      d.b.base = b + int64_t(k_begin) * ldb + n0;
+      d.b.bytes = (int64_t(p.K - k_begin) * ldb - n0) * 2;
+    }
+    d.c = C + (int64_t(g) * p.c_sg + int64_t(m0) * ldc + n0) * ESZ;
+    d.ldc = ldc;
+    d.c_bytes = (int64_t(p.M - m0) * ldc - n0) * ESZ;
+    d.klen = k_hi > k_begin ? k_hi - k_begin : 0;
+    d.row_rel0 = m0 - __builtin_amdgcn_readfirstlane(tile.m_lo);
+    d.row_cnt = __builtin_amdgcn_readfirstlane(tile.m_hi) - __builtin_amdgcn_readfirstlane(tile.m_lo);
+    d.col_lo = gmm_max(__builtin_amdgcn_readfirstlane(tile.n_lo) - n0, 0);
+    d.col_hi = gmm_min(__builtin_amdgcn_readfirstlane(tile.n_hi) - n0, GMM_TILE_N);
+    gmm_tile_compute<A_TR, B_TR, OUT_F32>(d, lds_base, lane, wave);
+  }
+}
+
+template <int OUT_F32>
+int launch_asm(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
+  const dim3 grid(p.num_wg), block(256);
+  if (lay.a_kc && lay.b_kc)
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32>), grid, block, 0, stream, p);
+  else if (lay.a_kc && !lay.b_kc)
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32>), grid, block, 0, stream, p);
+  else if (!lay.a_kc && lay.b_kc)
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32>), grid, block, 0, stream, p);
+  return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, typename OutT>
 int launch_layout(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -279,8 +356,12 @@ void gmm_mfma_tile_shape(int config, int& bm, int& bn) {
 }
 
 int gmm_launch_mfma(GmmParams p, GmmLayout lay, int out_dtype, int config, int num_cus, hipStream_t stream) {
-  (void)config;
   p.num_wg = num_cus;
+  if (config == GMM_CFG_ASM_256x256) {
+    if (out_dtype == GMM_DT_BF16) return launch_asm<0>(p, lay, stream);
+    if (out_dtype == GMM_DT_F32) return launch_asm<1>(p, lay, stream);
+    return -1;
+  }
   if (out_dtype == GMM_DT_BF16) return launch_layout<256, 256, 2, 2, uint16_t>(p, lay, stream);
   if (out_dtype == GMM_DT_F32) return launch_layout<256, 256, 2, 2, float>(p, lay, stream);
   return -1;
