@@ -38,7 +38,23 @@ Registers (fixed):
   v[64:95]     temporaries
   inputs are pinned by the C++ wrapper to v[128:...] and s[36:...] (see TileRegs).
 """
+import os
 import sys
+
+# copies (of the 16 per K tile and wave) issued in: step 3 right after the barrier, then steps 0, 1, 2
+# of the next K tile; the tile must have landed at that tile's barrier (end of its step 2).
+COPY_SCHEDULE = tuple(int(x) for x in os.environ.get("GMM_GEN_COPY_SCHEDULE", "6,5,5,0").split(","))
+assert len(COPY_SCHEDULE) == 4 and sum(COPY_SCHEDULE) == 16
+
+# L2 prefetch distance in K tiles (0 = off): in step 2 of K tile kt every lane touches one cache line of
+# K tile kt + PREFETCH of each operand, so that the copies issued two tiles later hit in L2.
+PREFETCH = int(os.environ.get("GMM_GEN_PREFETCH", "0"))
+
+# timing experiments only (results are wrong with these on)
+DBG_NO_COPY = int(os.environ.get("GMM_GEN_DBG_NO_COPY", "0"))
+DBG_NO_BARRIER = int(os.environ.get("GMM_GEN_DBG_NO_BARRIER", "0"))
+DBG_NO_MASK = int(os.environ.get("GMM_GEN_DBG_NO_MASK", "0"))
+DBG_TIMING = int(os.environ.get("GMM_GEN_DBG_TIMING", "0"))  # phase timestamps in s[92:99] (extra asm output)
 
 PITCH = 272           # bytes per staged row of 128 bf16 (256 + 16: shifts banks per row)
 TR_BLOCK = 1088       # two k rows of 512 bytes + 64 bytes pad
@@ -56,6 +72,8 @@ V_VOA_TAIL, V_VOB_TAIL = 160, 168
 V_RA, V_RB = 176, 180  # fragment read addresses (4 + 4)
 V_EPI = 184            # 184: stage write addr, 185: stage read addr, 186: store voffset, 187: row - row_lo
 V_OOB = 188            # constant 0x80000000
+V_PF = 192             # 192: A prefetch offset, 193: B prefetch offset
+V_PFD = 96             # dummy destinations of the prefetch loads (96, 97)
 
 S_RA, S_RB, S_RC = 36, 40, 44   # buffer resources
 S_SC = 48                        # scalars s[48:55]
@@ -150,6 +168,10 @@ class Variant:
         if which == "head":
             vo = (V_VOA_HEAD if is_a else V_VOB_HEAD) + i
             src = vr(vo)
+        elif DBG_NO_COPY:
+            return []
+        elif DBG_NO_MASK:
+            src = vr((V_VOA if is_a else V_VOB) + i)
         else:
             vn = (V_VOA if is_a else V_VOB) + i
             vt = (V_VOA_TAIL if is_a else V_VOB_TAIL) + i
@@ -197,8 +219,13 @@ def gen_variant(v):
         e("s_cmp_ge_u32 %s, %s" % (sr(s_tile), sr(S_NK)))
         e("s_cselect_b64 %s, -1, 0" % sr(s_oob, 2))
 
+    def stamp(k):
+        if DBG_TIMING:
+            e("s_memrealtime %s" % sr(92 + 2 * k, 2))
+
     # ------------------------------------------------------------------ prologue
     e("; ---- prologue (%s)" % v.name)
+    stamp(0)
     e("v_mov_b32 %s, 0x80000000" % vr(V_OOB))
     e("s_sub_u32 %s, %s, 1" % (sr(s_last), sr(S_NK)))
     e("s_mov_b32 %s, 0" % sr(s_zero))
@@ -216,14 +243,16 @@ def gen_variant(v):
     tile_masks(s_t1, s_tail1, s_oob1)
     e("s_mov_b32 %s, %s" % (sr(s_ka1), sr(S_ASTEP)))
     e("s_mov_b32 %s, %s" % (sr(s_kb1), sr(S_BSTEP)))
-    for n in range(6):
-        for ins in v.dma(n, 1, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + n):
+    c3, c0, c1, c2 = COPY_SCHEDULE
+    for n in range(c3):
+        for ins in v.dma(n, 1, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)):
             e(ins)
     # zero the accumulators while the copies fly
     for r in range(256):
         e("v_accvgpr_write_b32 a%d, 0" % r)
-    e("s_waitcnt vmcnt(6)")
+    e("s_waitcnt vmcnt(%d)" % c3)
     e("s_barrier")
+    stamp(1)
     for ins in v.frag_reads(0, 0, 0):
         e(ins)
     e("s_mov_b32 %s, 0" % sr(s_kt))
@@ -247,23 +276,33 @@ def gen_variant(v):
         # step 0: MFMA set 0, read step 1 -> set 1, copies 6..10 of tile kt+1 -> other buffer
         e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 1, 1)]
-        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(6, 11)]
+        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)]
         interleave(e, v.mfmas(0), side)
         # step 1
         e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 2, 0)]
-        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(11, 16)]
+        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)]
         interleave(e, v.mfmas(1), side)
         # step 2
         e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 3, 1)]
+        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, 16)]
+        npf = 0
+        if PREFETCH:
+            e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), PREFETCH))
+            e("s_mul_i32 %s, %s, %s" % (sr(sT + 16), sr(s_t1), sr(S_ASTEP)))
+            e("s_mul_i32 %s, %s, %s" % (sr(sT + 17), sr(s_t1), sr(S_BSTEP)))
+            side.append(["buffer_load_dword %s, %s, %s, %s offen" % (vr(V_PFD), vr(V_PF), sr(S_RA, 4), sr(sT + 16))])
+            side.append(["buffer_load_dword %s, %s, %s, %s offen" % (vr(V_PFD + 1), vr(V_PF + 1), sr(S_RB, 4), sr(sT + 17))])
+            npf = 2
         interleave(e, v.mfmas(0), side)
         # tile kt+1 has landed for this wave; after the barrier for all, and `buf` is free
-        e("s_waitcnt vmcnt(0) lgkmcnt(0)")
-        e("s_barrier")
+        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % npf)
+        if not DBG_NO_BARRIER:
+            e("s_barrier")
         # step 3: MFMA set 1, read step 0 of the next tile -> set 0, copies 0..5 of tile kt+2 -> buf
         side = [[x] for x in v.frag_reads(nb, 0, 0)]
-        side += [v.dma(n, buf, "loop", s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, 6)]
+        side += [v.dma(n, buf, "loop", s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, c3)]
         interleave(e, v.mfmas(1), side)
         e("s_add_u32 %s, %s, 1" % (sr(s_kt), sr(s_kt)))
 
@@ -278,6 +317,7 @@ def gen_variant(v):
 
     # ------------------------------------------------------------------ epilogue
     e("; ---- epilogue")
+    stamp(2)
     e("s_waitcnt vmcnt(0) lgkmcnt(0)")
     e("s_nop 15")
     e("s_nop 15")
@@ -346,6 +386,7 @@ def gen_variant(v):
                         e("s_and_b64 vcc, %s, %s" % (sr(S_T + 32, 2), sr(S_T + 24 + 2 * j, 2)))
                         e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(t + 8 + (k % 8)), vr(V_OOB), vr(V_EPI + 2)))
                         e("buffer_store_dword %s, %s, %s, %s offen offset:%d" % (vr(b), vr(t + 8 + (k % 8)), sr(S_RC, 4), sr(S_T + 16), 128 * j))
+    stamp(3)
     e("s_waitcnt lgkmcnt(0)")
     e("s_barrier")
     return e
@@ -353,7 +394,7 @@ def gen_variant(v):
 
 def clobbers():
     c = ["memory", "vcc", "scc"]
-    c += ["v%d" % i for i in range(0, 96)] + ["v%d" % V_OOB]
+    c += ["v%d" % i for i in range(0, 98)] + ["v%d" % V_OOB]
     c += ["a%d" % i for i in range(256)]
     c += ["s%d" % i for i in range(S_T, S_T + 34)]
     return ", ".join('"%s"' % x for x in c)
@@ -374,13 +415,13 @@ def main():
                 v = Variant(a_tr, b_tr, f32)
                 e = gen_variant(v)
                 out.append("")
-                out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d>(const GmmTileRegs& r) {" % (a_tr, b_tr, f32))
+                out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32))
                 out.append("  asm volatile(")
                 out.append(e.text())
-                out.append("      :")
+                out.append('      : "={s[92:99]}"(r.stamps)' if DBG_TIMING else "      :")
                 out.append('      : "{v[128:135]}"(r.voa_head), "{v[136:143]}"(r.vob_head), "{v[144:151]}"(r.voa), "{v[152:159]}"(r.vob),')
                 out.append('        "{v[160:167]}"(r.voa_tail), "{v[168:175]}"(r.vob_tail), "{v[176:179]}"(r.ra_addr), "{v[180:183]}"(r.rb_addr),')
-                out.append('        "{v[184:187]}"(r.epi), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
+                out.append('        "{v[184:187]}"(r.epi), "{v[192:193]}"(r.pf), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
                 out.append("      : %s);" % clobbers())
                 out.append("}")
     sys.stdout.write("\n".join(out) + "\n")

@@ -265,6 +265,7 @@ template <int A_TR, int B_TR, int OUT_F32>
 __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[gmm_tile_lds_bytes<A_TR, B_TR>()];
   __shared__ int32_t cum[GMM_MAX_GROUPS + 1];
+  __shared__ int32_t tiles[256][12];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
@@ -278,43 +279,63 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
   const int ldb = int(B_TR ? p.b_sk : p.b_sn);
   const int ldc = int(p.c_sm);
 
-  for (int t = blockIdx.x; t < total; t += gridDim.x) {
-    const int tt = p.xcd_remap ? gmm_xcd_remap(t, total, gridDim.x) : t;
-    const GmmTile tile = gmm_locate_tile(p, cum, tt, GMM_TILE_M, GMM_TILE_N);
-    const int g = __builtin_amdgcn_readfirstlane(tile.g);
-    const int m0 = __builtin_amdgcn_readfirstlane(tile.m0), n0 = __builtin_amdgcn_readfirstlane(tile.n0);
-    const int k_lo = __builtin_amdgcn_readfirstlane(tile.k_lo), k_hi = __builtin_amdgcn_readfirstlane(tile.k_hi);
-    // the copies move 16-byte chunks along K for an operand that is contiguous along K
-    const int k_begin = (A_TR && B_TR) ? k_lo : (k_lo & ~7);
-    const uint16_t* a = A + int64_t(g) * p.a_sg;
-    const uint16_t* b = B + int64_t(g) * p.b_sg;
+  // This workgroup's tiles are blockIdx.x, blockIdx.x + gridDim.x, ...  Locating a tile (binary search
+  // over the groups, reads of offs, integer divisions) costs microseconds, so the 256 threads locate
+  // the next 256 tiles of the workgroup at once and leave them in LDS for the tile loop to pick up.
+  for (int first = 0;; first += 256) {
+    const int64_t mine = int64_t(blockIdx.x) + int64_t(first + tid) * gridDim.x;
+    if (mine < total) {
+      const int t = int(mine);
+      const int tt = p.xcd_remap ? gmm_xcd_remap(t, total, gridDim.x) : t;
+      const GmmTile tile = gmm_locate_tile_divergent(p, cum, tt, GMM_TILE_M, GMM_TILE_N);
+      int32_t* d = tiles[tid];
+      d[0] = tile.g; d[1] = tile.m0; d[2] = tile.n0; d[3] = tile.m_lo; d[4] = tile.m_hi;
+      d[5] = tile.n_lo; d[6] = tile.n_hi; d[7] = tile.k_lo; d[8] = tile.k_hi;
+    }
+    __syncthreads();
+    const int64_t left = (int64_t(total) - blockIdx.x + gridDim.x - 1) / gridDim.x - first;  // tiles of this workgroup from `first` on
+    const int here = left < 256 ? int(left) : 256;
+    for (int j = 0; j < here; ++j) {
+      const int32_t* d = tiles[j];
+      const int g = __builtin_amdgcn_readfirstlane(d[0]);
+      const int m0 = __builtin_amdgcn_readfirstlane(d[1]), n0 = __builtin_amdgcn_readfirstlane(d[2]);
+      const int m_lo = __builtin_amdgcn_readfirstlane(d[3]), m_hi = __builtin_amdgcn_readfirstlane(d[4]);
+      const int n_lo = __builtin_amdgcn_readfirstlane(d[5]), n_hi = __builtin_amdgcn_readfirstlane(d[6]);
+      const int k_lo = __builtin_amdgcn_readfirstlane(d[7]), k_hi = __builtin_amdgcn_readfirstlane(d[8]);
+      // the copies move 16-byte chunks along K for an operand that is contiguous along K
+      const int k_begin = (A_TR && B_TR) ? k_lo : (k_lo & ~7);
+      const uint16_t* a = A + int64_t(g) * p.a_sg;
+      const uint16_t* b = B + int64_t(g) * p.b_sg;
 
-    GmmTileDesc d;
-    d.a.ld = lda;
-    d.b.ld = ldb;
-    if (!A_TR) {
-      d.a.base = a + int64_t(m0) * lda + k_begin;
-      d.a.bytes = (int64_t(p.M - m0) * lda - k_begin) * 2;
-    } else {
-      d.a.base = a + int64_t(k_begin) * lda + m0;
-      d.a.bytes = (int64_t(p.K - k_begin) * lda - m0) * 2;
+      GmmTileDesc dsc;
+      dsc.a.ld = lda;
+      dsc.b.ld = ldb;
+      if (!A_TR) {
+        dsc.a.base = a + int64_t(m0) * lda + k_begin;
+        dsc.a.bytes = (int64_t(p.M - m0) * lda - k_begin) * 2;
+      } else {
+        dsc.a.base = a + int64_t(k_begin) * lda + m0;
+        dsc.a.bytes = (int64_t(p.K - k_begin) * lda - m0) * 2;
+      }
+      if (!B_TR) {
+        dsc.b.base = b + int64_t(n0) * ldb + k_begin;
+        dsc.b.bytes = (int64_t(p.N - n0) * ldb - k_begin) * 2;
+      } else {
+        dsc.b.base = b + int64_t(k_begin) * ldb + n0;
+        dsc.b.bytes = (int64_t(p.K - k_begin) * ldb - n0) * 2;
+      }
+      dsc.c = C + (int64_t(g) * p.c_sg + int64_t(m0) * ldc + n0) * ESZ;
+      dsc.ldc = ldc;
+      dsc.c_bytes = (int64_t(p.M - m0) * ldc - n0) * ESZ;
+      dsc.klen = k_hi > k_begin ? k_hi - k_begin : 0;
+      dsc.row_rel0 = m0 - m_lo;
+      dsc.row_cnt = m_hi - m_lo;
+      dsc.col_lo = gmm_max(n_lo - n0, 0);
+      dsc.col_hi = gmm_min(n_hi - n0, GMM_TILE_N);
+      gmm_tile_compute<A_TR, B_TR, OUT_F32>(dsc, lds_base, lane, wave);
     }
-    if (!B_TR) {
-      d.b.base = b + int64_t(n0) * ldb + k_begin;
-      d.b.bytes = (int64_t(p.N - n0) * ldb - k_begin) * 2;
-    } else {
-      d.b.base = b + int64_t(k_begin) * ldb + n0;
-      d.b.bytes = (int64_t(p.K - k_begin) * ldb - n0) * 2;
-    }
-    d.c = C + (int64_t(g) * p.c_sg + int64_t(m0) * ldc + n0) * ESZ;
-    d.ldc = ldc;
-    d.c_bytes = (int64_t(p.M - m0) * ldc - n0) * ESZ;
-    d.klen = k_hi > k_begin ? k_hi - k_begin : 0;
-    d.row_rel0 = m0 - __builtin_amdgcn_readfirstlane(tile.m_lo);
-    d.row_cnt = __builtin_amdgcn_readfirstlane(tile.m_hi) - __builtin_amdgcn_readfirstlane(tile.m_lo);
-    d.col_lo = gmm_max(__builtin_amdgcn_readfirstlane(tile.n_lo) - n0, 0);
-    d.col_hi = gmm_min(__builtin_amdgcn_readfirstlane(tile.n_hi) - n0, GMM_TILE_N);
-    gmm_tile_compute<A_TR, B_TR, OUT_F32>(d, lds_base, lane, wave);
+    if (left <= 256) break;
+    __syncthreads();  // everyone is done with this batch of located tiles
   }
 }
 

@@ -7,6 +7,7 @@
 
 typedef int gmm_v4i __attribute__((ext_vector_type(4)));
 typedef int gmm_v8i __attribute__((ext_vector_type(8)));
+typedef int gmm_v2i __attribute__((ext_vector_type(2)));
 
 struct GmmTileRegs {
   gmm_v8i voa_head, vob_head;  // copy offsets of K tile 0 (first/last chunk masks applied)
@@ -14,12 +15,14 @@ struct GmmTileRegs {
   gmm_v8i voa_tail, vob_tail;  // copy offsets of the last K tile
   gmm_v4i ra_addr, rb_addr;    // LDS fragment read addresses
   gmm_v4i epi;                 // epilogue: per-lane addresses (see gen_tile_asm.py)
+  gmm_v2i pf;                  // L2 prefetch offsets of this lane for A and B
   gmm_v4i rsrc_a, rsrc_b, rsrc_c;
   gmm_v8i scal;                // nk, a_step, b_step, lds_base, row_cnt, c_step, n_valid, wave
+  gmm_v8i stamps;              // timing builds only: four 64-bit s_memrealtime stamps
 };
 
 template <int A_TR, int B_TR, int OUT_F32>
-__device__ __forceinline__ void gmm_tile_asm(const GmmTileRegs& r);
+__device__ __forceinline__ void gmm_tile_asm(GmmTileRegs& r);
 
 #include "gmm_tile_asm.inc"
 
@@ -87,7 +90,8 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int
 }
 
 template <int A_TR, int B_TR, int OUT_F32>
-__device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave) {
+__device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave,
+                                                 gmm_v8i* stamps = nullptr) {
   constexpr int A_STAGE = A_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE;
   const int wm = wave & 1, wn = wave >> 1;
   const int nk = (t.klen + GMM_TILE_K - 1) / GMM_TILE_K;
@@ -111,6 +115,9 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
       r.rb_addr[s] = lds_base + 2 * A_STAGE + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wn * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
     }
   }
+  // L2 prefetch: 256 cache lines per operand and K tile, one per lane
+  r.pf[0] = A_TR ? (wave * 16 + (lane >> 2)) * t.a.ld * 2 + (lane & 3) * 128 : (wave * 64 + lane) * t.a.ld * 2;
+  r.pf[1] = B_TR ? (wave * 16 + (lane >> 2)) * t.b.ld * 2 + (lane & 3) * 128 : (wave * 64 + lane) * t.b.ld * 2;
   int c_step, n_valid = 0;
   if (!OUT_F32) {
     const int row_t = wm * 128 + (lane >> 4), col_t = wn * 128 + (lane & 15) * 8;
@@ -137,4 +144,5 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   gmm_v8i sc = {nk, a_step, b_step, (int)lds_base, t.row_cnt, c_step, n_valid, wave};
   r.scal = sc;
   gmm_tile_asm<A_TR, B_TR, OUT_F32>(r);
+  if (stamps) *stamps = r.stamps;
 }
