@@ -43,7 +43,7 @@ import sys
 
 # copies (of the 16 per K tile and wave) issued in: step 3 right after the barrier, then steps 0, 1, 2
 # of the next K tile; the tile must have landed at that tile's barrier (end of its step 2).
-COPY_SCHEDULE = tuple(int(x) for x in os.environ.get("GMM_GEN_COPY_SCHEDULE", "6,5,5,0").split(","))
+COPY_SCHEDULE = tuple(int(x) for x in os.environ.get("GMM_GEN_COPY_SCHEDULE", "8,8,0,0").split(","))
 assert len(COPY_SCHEDULE) == 4 and sum(COPY_SCHEDULE) == 16
 
 # L2 prefetch distance in K tiles (0 = off): in step 2 of K tile kt every lane touches one cache line of
@@ -74,6 +74,8 @@ V_EPI = 184            # 184: stage write addr, 185: stage read addr, 186: store
 V_OOB = 188            # constant 0x80000000
 V_PF = 192             # 192: A prefetch offset, 193: B prefetch offset
 V_PFD = 96             # dummy destinations of the prefetch loads (96, 97)
+V_FIX = 196            # 196: A first-chunk addr, 197: A last-chunk addr, 198 / 199: same for B (buffer 0)
+S_MASK = 28            # s[28:31] keep-mask of the first chunk of the k range, s[32:35] of the last chunk
 
 S_RA, S_RB, S_RC = 36, 40, 44   # buffer resources
 S_SC = 48                        # scalars s[48:55]
@@ -184,6 +186,30 @@ class Variant:
         return out
 
 
+def fixup(e, v, which, buf):
+    """Zero the k elements outside the group's range in one 16-byte chunk per row (row = thread id) of
+    every operand that is contiguous along K.  which: 0 = first chunk of K tile 0, 1 = last chunk."""
+    for is_a in (True, False):
+        tr = v.a_tr if is_a else v.b_tr
+        if tr:
+            continue
+        stage = v.a_stage if is_a else v.b_stage
+        addr = V_FIX + (0 if is_a else 2) + which
+        t = V_TMP + (0 if is_a else 4)
+        e("ds_read_b128 %s, %s offset:%d" % (vr(t, 4), vr(addr), buf * stage))
+    e("s_waitcnt lgkmcnt(0)")
+    for is_a in (True, False):
+        tr = v.a_tr if is_a else v.b_tr
+        if tr:
+            continue
+        stage = v.a_stage if is_a else v.b_stage
+        addr = V_FIX + (0 if is_a else 2) + which
+        t = V_TMP + (0 if is_a else 4)
+        for w in range(4):
+            e("v_and_b32 %s, %s, %s" % (vr(t + w), sr(S_MASK + 4 * which + w), vr(t + w)))
+        e("ds_write_b128 %s, %s offset:%d" % (vr(addr), vr(t, 4), buf * stage))
+
+
 def interleave(e, mfmas, side_groups):
     """Emit 16 MFMAs with the side groups spread between them (one group after each MFMA, in order)."""
     n = len(mfmas)
@@ -227,12 +253,16 @@ def gen_variant(v):
     e("; ---- prologue (%s)" % v.name)
     stamp(0)
     e("v_mov_b32 %s, 0x80000000" % vr(V_OOB))
+    # s[S_SPARE] = wave id | fix-up flags << 8 (bit 0: first chunk of the k range is partial, bit 1: last chunk)
+    s_flags = sT + 18
+    e("s_lshr_b32 %s, %s, 8" % (sr(s_flags), sr(S_SPARE)))
+    e("s_and_b32 %s, %s, 0xff" % (sr(sT + 19), sr(S_SPARE)))
     e("s_sub_u32 %s, %s, 1" % (sr(s_last), sr(S_NK)))
     e("s_mov_b32 %s, 0" % sr(s_zero))
     # wave part of the LDS copy destinations: wave id is in s[S_SPARE]
-    e("s_mul_i32 %s, %s, %d" % (sr(s_waveA), sr(S_SPARE), 8 * (TR_BLOCK if v.a_tr else 1024)))
+    e("s_mul_i32 %s, %s, %d" % (sr(s_waveA), sr(sT + 19), 8 * (TR_BLOCK if v.a_tr else 1024)))
     e("s_add_u32 %s, %s, %s" % (sr(s_waveA), sr(s_waveA), sr(S_LDS)))
-    e("s_mul_i32 %s, %s, %d" % (sr(s_waveB), sr(S_SPARE), 8 * (TR_BLOCK if v.b_tr else 1024)))
+    e("s_mul_i32 %s, %s, %d" % (sr(s_waveB), sr(sT + 19), 8 * (TR_BLOCK if v.b_tr else 1024)))
     e("s_add_u32 %s, %s, %s" % (sr(s_waveB), sr(s_waveB), sr(S_LDS)))
     # tile 0 -> buffer 0 (head offsets)
     for n in range(16):
@@ -253,6 +283,25 @@ def gen_variant(v):
     e("s_waitcnt vmcnt(%d)" % c3)
     e("s_barrier")
     stamp(1)
+    has_kc = not (v.a_tr and v.b_tr)
+    if has_kc:
+        # partial first / last chunk of a jagged k range (tile 0 is also the last tile when nk == 1)
+        e("s_cmp_eq_u32 %s, 0" % sr(s_flags))
+        e("s_cbranch_scc1 L_nofix0_%s" % L)
+        e("s_bitcmp1_b32 %s, 0" % sr(s_flags))
+        e("s_cbranch_scc0 L_nohead_%s" % L)
+        fixup(e, v, 0, 0)
+        e("s_waitcnt lgkmcnt(0)")
+        e.label("L_nohead_%s" % L)
+        e("s_bitcmp1_b32 %s, 1" % sr(s_flags))
+        e("s_cbranch_scc0 L_notail0_%s" % L)
+        e("s_cmp_eq_u32 %s, 1" % sr(S_NK))
+        e("s_cbranch_scc0 L_notail0_%s" % L)
+        fixup(e, v, 1, 0)
+        e.label("L_notail0_%s" % L)
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_barrier")
+        e.label("L_nofix0_%s" % L)
     for ins in v.frag_reads(0, 0, 0):
         e(ins)
     e("s_mov_b32 %s, 0" % sr(s_kt))
@@ -300,6 +349,17 @@ def gen_variant(v):
         e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % npf)
         if not DBG_NO_BARRIER:
             e("s_barrier")
+        if not (v.a_tr and v.b_tr):
+            # the tile that has just landed is the last one and its last chunk is partial
+            e("s_add_u32 %s, %s, 1" % (sr(s_t1), sr(s_kt)))
+            e("s_cmp_eq_u32 %s, %s" % (sr(s_t1), sr(s_last)))
+            e("s_cbranch_scc0 L_nofix%d_%s" % (buf + 1, L))
+            e("s_bitcmp1_b32 %s, 1" % sr(sT + 18))
+            e("s_cbranch_scc0 L_nofix%d_%s" % (buf + 1, L))
+            fixup(e, v, 1, nb)
+            e("s_waitcnt lgkmcnt(0)")
+            e("s_barrier")
+            e.label("L_nofix%d_%s" % (buf + 1, L))
         # step 3: MFMA set 1, read step 0 of the next tile -> set 0, copies 0..5 of tile kt+2 -> buf
         side = [[x] for x in v.frag_reads(nb, 0, 0)]
         side += [v.dma(n, buf, "loop", s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, c3)]
@@ -421,7 +481,7 @@ def main():
                 out.append('      : "={s[92:99]}"(r.stamps)' if DBG_TIMING else "      :")
                 out.append('      : "{v[128:135]}"(r.voa_head), "{v[136:143]}"(r.vob_head), "{v[144:151]}"(r.voa), "{v[152:159]}"(r.vob),')
                 out.append('        "{v[160:167]}"(r.voa_tail), "{v[168:175]}"(r.vob_tail), "{v[176:179]}"(r.ra_addr), "{v[180:183]}"(r.rb_addr),')
-                out.append('        "{v[184:187]}"(r.epi), "{v[192:193]}"(r.pf), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
+                out.append('        "{v[184:187]}"(r.epi), "{v[192:193]}"(r.pf), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
                 out.append("      : %s);" % clobbers())
                 out.append("}")
     sys.stdout.write("\n".join(out) + "\n")

@@ -66,7 +66,6 @@ bool mfma_eligible(const Problem& pr, GmmLayout& lay, int& align) {
 bool asm_tile_eligible(const Problem& pr, const GmmLayout& lay) {
   const GmmParams& p = pr.p;
   if (p.jag == GMM_JAG_N) return false;                           // jagged columns: element-masked stores
-  if (p.jag == GMM_JAG_K && (lay.a_kc || lay.b_kc)) return false;  // unaligned k ranges need element masks
   if (p.c_sn != 1) return false;
   const int64_t lda = lay.a_kc ? p.a_sm : p.a_sk, ldb = lay.b_kc ? p.b_sn : p.b_sk, ldc = p.c_sm;
   const int64_t ld_max = int64_t(1) << 22;

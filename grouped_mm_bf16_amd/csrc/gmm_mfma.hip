@@ -327,7 +327,8 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       dsc.c = C + (int64_t(g) * p.c_sg + int64_t(m0) * ldc + n0) * ESZ;
       dsc.ldc = ldc;
       dsc.c_bytes = (int64_t(p.M - m0) * ldc - n0) * ESZ;
-      dsc.klen = k_hi > k_begin ? k_hi - k_begin : 0;
+      dsc.klen = k_hi > k_lo ? k_hi - k_begin : 0;
+      dsc.khead = k_lo - k_begin;
       dsc.row_rel0 = m0 - m_lo;
       dsc.row_cnt = m_hi - m_lo;
       dsc.col_lo = gmm_max(n_lo - n0, 0);

@@ -16,6 +16,8 @@ struct GmmTileRegs {
   gmm_v4i ra_addr, rb_addr;    // LDS fragment read addresses
   gmm_v4i epi;                 // epilogue: per-lane addresses (see gen_tile_asm.py)
   gmm_v2i pf;                  // L2 prefetch offsets of this lane for A and B
+  gmm_v4i fix;                 // LDS addresses of this thread's row in the first / last k chunk (A, A, B, B)
+  gmm_v8i masks;               // keep-masks of the first and of the last 16-byte k chunk
   gmm_v4i rsrc_a, rsrc_b, rsrc_c;
   gmm_v8i scal;                // nk, a_step, b_step, lds_base, row_cnt, c_step, n_valid, wave
   gmm_v8i stamps;              // timing builds only: four 64-bit s_memrealtime stamps
@@ -40,7 +42,9 @@ __device__ __forceinline__ gmm_v4i gmm_make_rsrc(const void* p, long long bytes)
   const unsigned long long a = (unsigned long long)p;
   if (bytes < 0) bytes = 0;
   if (bytes > 0x7fffffffLL) bytes = 0x7fffffffLL;
-  gmm_v4i r = {(int)(unsigned)a, (int)(unsigned)((a >> 32) & 0xffffu), (int)bytes, 0x00020000};
+  gmm_v4i r = {__builtin_amdgcn_readfirstlane((int)(unsigned)a),
+               __builtin_amdgcn_readfirstlane((int)(unsigned)((a >> 32) & 0xffffu)),
+               __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
   return r;
 }
 
@@ -61,14 +65,15 @@ struct GmmTileDesc {
   void* c;               // element (m0, n0) of the output
   int ldc;
   long long c_bytes;     // from c to the end of the output storage
-  int klen;
+  int klen;              // k elements from k_begin that count ...
+  int khead;             // ... of which the first khead are before the group's range (0..7) and read as zero
   int row_rel0;          // m0 - m_lo   (may be negative: rows before m_lo are not stored)
   int row_cnt;           // m_hi - m_lo
   int col_lo, col_hi;    // columns [col_lo, col_hi) of the tile are stored (relative to n0)
 };
 
 template <int TR>
-__device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int klen, int nk,
+__device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int klen, int khead, int nk,
                                                  gmm_v8i& head, gmm_v8i& full, gmm_v8i& tail) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -83,9 +88,11 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int
       k = 8 * (blk >> 2) + (blk & 3) + 4 * (lane >> 5);
       vo = k * ld * 2 + (lane & 31) * 16;
     }
+    // whole k rows before the range are skipped (transposed layout); inside a chunk the fix-up masks them
+    const bool before = TR && k < khead;
     full[i] = vo;
-    head[i] = (k < klen) ? vo : (int)GMM_OOB;
-    tail[i] = ((nk - 1) * GMM_TILE_K + k < klen) ? vo : (int)GMM_OOB;
+    head[i] = (k < klen && !before) ? vo : (int)GMM_OOB;
+    tail[i] = ((nk - 1) * GMM_TILE_K + k < klen && !(before && nk == 1)) ? vo : (int)GMM_OOB;
   }
 }
 
@@ -96,8 +103,8 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   const int wm = wave & 1, wn = wave >> 1;
   const int nk = (t.klen + GMM_TILE_K - 1) / GMM_TILE_K;
   GmmTileRegs r;
-  gmm_copy_offsets<A_TR>(lane, wave, t.a.ld, t.klen, nk, r.voa_head, r.voa, r.voa_tail);
-  gmm_copy_offsets<B_TR>(lane, wave, t.b.ld, t.klen, nk, r.vob_head, r.vob, r.vob_tail);
+  gmm_copy_offsets<A_TR>(lane, wave, t.a.ld, t.klen, t.khead, nk, r.voa_head, r.voa, r.voa_tail);
+  gmm_copy_offsets<B_TR>(lane, wave, t.b.ld, t.klen, t.khead, nk, r.vob_head, r.vob, r.vob_tail);
   const int q = lane >> 4, ii = lane & 15;
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
@@ -141,8 +148,28 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   r.rsrc_c = gmm_make_rsrc(t.c, t.c_bytes);
   const int a_step = A_TR ? GMM_TILE_K * t.a.ld * 2 : GMM_TILE_K * 2;
   const int b_step = B_TR ? GMM_TILE_K * t.b.ld * 2 : GMM_TILE_K * 2;
-  gmm_v8i sc = {nk, a_step, b_step, (int)lds_base, t.row_cnt, c_step, n_valid, wave};
-  r.scal = sc;
+  // partial first / last chunk of the k range (jagged contraction with an operand contiguous along K)
+  const int ktail = t.klen & 7;
+  int flags = 0;
+  if (!(A_TR && B_TR)) flags = (t.khead ? 1 : 0) | (ktail ? 2 : 0);
+  {
+    const int row = threadIdx.x;                      // one row of each 256-row operand tile per thread
+    const int c_last = ((t.klen - 1) & (GMM_TILE_K - 1)) >> 3;
+    r.fix[0] = lds_base + row * 128 + ((0 ^ gmm_swz(row)) << 4);
+    r.fix[1] = lds_base + row * 128 + ((c_last ^ gmm_swz(row)) << 4);
+    r.fix[2] = r.fix[0] + 2 * A_STAGE;
+    r.fix[3] = r.fix[1] + 2 * A_STAGE;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const unsigned h0 = (2 * w >= t.khead) ? 0x0000ffffu : 0u, h1 = (2 * w + 1 >= t.khead) ? 0xffff0000u : 0u;
+      const unsigned t0 = (2 * w < ktail) ? 0x0000ffffu : 0u, t1 = (2 * w + 1 < ktail) ? 0xffff0000u : 0u;
+      r.masks[w] = __builtin_amdgcn_readfirstlane((int)(h0 | h1));
+      r.masks[4 + w] = __builtin_amdgcn_readfirstlane((int)(t0 | t1));
+    }
+  }
+  const int sc[8] = {nk, a_step, b_step, (int)lds_base, t.row_cnt, c_step, n_valid, wave | (flags << 8)};
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r.scal[i] = __builtin_amdgcn_readfirstlane(sc[i]);
   gmm_tile_asm<A_TR, B_TR, OUT_F32>(r);
   if (stamps) *stamps = r.stamps;
 }
