@@ -28,6 +28,9 @@ if ROOT not in sys.path:
 METRIC = "TFLOP/s + % bf16 MFMA peak, 2D×3D MoE G=8 K=4096 N=14336, 1 GPU"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the copy-kernel
+# calibration); see profiles/.  None where no profile has been taken.
+MEASURED_TRAFFIC = {"mixtral": None, "fine": None, "batched": None, "batched_colmajor": None, "kgrouped": None}
 
 
 def load_sizes(key):
@@ -144,7 +147,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="mixtral",
-                    choices=["mixtral", "fine", "batched", "batched_colmajor", "kgrouped"])
+                    choices=["mixtral", "fine", "batched", "batched_colmajor", "kgrouped", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--path", default="auto", choices=["auto", "mfma", "generic"])
     args = ap.parse_args()
@@ -160,6 +163,22 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "copy":
+        # plain 1 GiB device copy: the known-size kernel that calibrates rocprof's FETCH_SIZE / WRITE_SIZE
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / args.steps * 1e3
+        print(json.dumps({"metric": "device copy of 1 GiB (calibration)", "value": round(2 * (1 << 30) / ms / 1e6, 1),
+                          "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                          "ms_per_step": round(ms, 4), "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
+        return
     w = make_workload(args.workload, torch)
     a, b = w["a"].to(dev), w["b"].to(dev)
     if w.get("b_col"):
@@ -221,7 +240,7 @@ def main():
         "config": {"workload": w["desc"], "kernel_family": path,
                    "pct_bf16_mfma_peak": round(tflops / PEAK_BF16_TFLOPS * 100, 2)},
         "roofline": {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
                      "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(k_ms), 4),
                      "kernel_ms_median": round(statistics.median(k_ms), 4),
                      "algorithmic_flops": w["flops"], "algorithmic_bytes": w["bytes"]},
