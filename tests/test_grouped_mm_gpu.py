@@ -242,6 +242,36 @@ def test_fp32_epilogue_for_bf16_inputs_through_the_launcher():
         grouped_mm(a.to(DEV), b.to(DEV), offs=offs_of(sizes).to(DEV), out_dtype=torch.float32)
 
 
+def test_non_finite_values_stay_inside_their_group():
+    """Elements of a neighbouring group must never enter a product, not even multiplied by zero:
+    poison one group's rows / k range with NaN and Inf and check every other group is untouched."""
+    gen = torch.Generator().manual_seed(53)
+    sizes = [13, 70, 0, 131, 58]  # odd boundaries: k ranges start inside 16-byte chunks
+    offs, tot = offs_of(sizes), sum(sizes)
+    rng = oracle.group_ranges(offs.tolist())
+    # 2D x 2D (jagged contraction), row-major A (K contiguous) and row-major B
+    a, b = rnd(gen, 264, tot), rnd(gen, tot, 272)
+    s, e = rng[1]
+    a[:, s:e] = float("nan")
+    b[s:e, :] = float("inf")
+    for path, cfg in (("mfma", 1), ("mfma", 0), ("generic", -1)):
+        with K_.forced_path(path), K_.forced_mfma_config(cfg):
+            out = run_poisoned(K_.grouped_mm_2d2d, a, b, offs, (len(sizes), 264, 272), torch.float32)
+        want = oracle.grouped_mm(a, b, offs, out_dtype=torch.float32)
+        for g in (0, 2, 3, 4):
+            assert torch.isfinite(out[g]).all(), (path, cfg, g)
+            torch.testing.assert_close(out[g], want[g], rtol=1.6e-2, atol=1e-2 * (131 / 64) ** 0.5)
+        assert not torch.isfinite(out[1]).any()
+    # 2D x 3D (jagged rows): a poisoned group poisons only its own rows
+    a, b = rnd(gen, tot, 64), rnd(gen, len(sizes), 64, 48)
+    a[s:e] = float("nan")
+    out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs, (tot, 48), torch.bfloat16)
+    assert torch.isnan(out[s:e].float()).all()
+    keep = torch.ones(tot, dtype=torch.bool)
+    keep[s:e] = False
+    assert torch.isfinite(out[keep].float()).all()
+
+
 # ------------------------------------------------------------------ host rules on real tensors
 def test_rules_on_gpu_tensors_and_shortcuts():
     a = torch.randn(8, 16, device=DEV, dtype=torch.bfloat16)
