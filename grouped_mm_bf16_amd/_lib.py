@@ -35,6 +35,8 @@ SIGNATURES = {
     "gmm_last_mfma_config": (ctypes.c_int, []),
     "gmm_set_xcd_remap": (ctypes.c_int, [ctypes.c_int]),
     "gmm_host_tile_list": (_i64, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _i64]),
+    "gmm_host_tile_list2": (_i64, [_vp] + [_i32] * 11 + [_vp, _i64]),
+    "gmm_set_tile_heights": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
 }
 
 _lock = threading.Lock()

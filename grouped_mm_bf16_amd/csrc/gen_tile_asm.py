@@ -74,6 +74,8 @@ V_EPI = 184            # 184: stage write addr, 185: stage read addr, 186: store
 V_OOB = 188            # constant 0x80000000
 V_PF = 192             # 192: A prefetch offset, 193: B prefetch offset
 V_PFD = 96             # dummy destinations of the prefetch loads (96, 97)
+STAGES_SHORT = int(os.environ.get('GMM_GEN_STAGES_SHORT', '2'))  # LDS buffers of the 128- and 64-row tiles
+V_BUFA, V_BUFB = 98, 110  # three-buffer variants: fragment addresses per (buffer, step), 12 + 12 registers
 V_FIX = 196            # 196: A first-chunk addr, 197: A last-chunk addr, 198 / 199: same for B (buffer 0)
 S_MASK = 28            # s[28:31] keep-mask of the first chunk of the k range, s[32:35] of the last chunk
 
@@ -110,30 +112,46 @@ def sr(base, n=1):
 
 
 class Variant:
-    def __init__(self, a_tr, b_tr, out_f32):
-        self.a_tr, self.b_tr, self.out_f32 = a_tr, b_tr, out_f32
-        self.a_stage = TR_STAGE if a_tr else KC_STAGE
+    """tm = MFMA block rows per wave: the tile is 64 tm rows (256 / 128 / 64) by 256 columns."""
+
+    def __init__(self, a_tr, b_tr, out_f32, tm=4):
+        self.a_tr, self.b_tr, self.out_f32, self.tm = a_tr, b_tr, out_f32, tm
+        assert tm in (1, 2, 4) and (tm == 4 or not a_tr)
+        self.na = 2 * tm                 # copies of the A tile per wave and K tile (B: always 8)
+        self.ncopy = self.na + 8
+        c3 = (self.ncopy + 1) // 2 if COPY_SCHEDULE == (8, 8, 0, 0) else None
+        self.sched = (c3, self.ncopy - c3, 0, 0) if c3 is not None else COPY_SCHEDULE
+        # LDS buffers per operand: 2 for the 256-row tile (LDS is full), 3 for the shorter ones, whose K
+        # tiles are short of MFMA work and would otherwise wait on memory latency every K tile
+        self.stages = STAGES_SHORT if tm < 4 else 2
+        self.a_stage = TR_STAGE if a_tr else (64 * tm * 128 if self.stages == 3 else KC_STAGE)
         self.b_stage = TR_STAGE if b_tr else KC_STAGE
-        self.b_base = 2 * self.a_stage          # LDS offset of B buffer 0
+        self.b_base = self.stages * self.a_stage   # LDS offset of B buffer 0
         self.swap = not out_f32                  # bf16: lanes own 4 consecutive columns
-        self.name = "%s%s_%s" % ("t" if a_tr else "k", "t" if b_tr else "k", "f32" if out_f32 else "bf16")
+        self.name = "%s%s_%s_m%d" % ("t" if a_tr else "k", "t" if b_tr else "k", "f32" if out_f32 else "bf16", 64 * tm)
 
     # -- fragment reads of k16 step `s` of buffer `buf` into register set `st`; returns list of instr
     def frag_reads(self, buf, s, st):
         out = []
-        for op, tr, vbase, vaddr, stage, lbase in (
-            ("A", self.a_tr, V_AF[st], V_RA, self.a_stage, 0),
-            ("B", self.b_tr, V_BF[st], V_RB, self.b_stage, 0),
+        for op, tr, vbase, vaddr, vbuf, stage, nblk in (
+            ("A", self.a_tr, V_AF[st], V_RA, V_BUFA, self.a_stage, self.tm),
+            ("B", self.b_tr, V_BF[st], V_RB, V_BUFB, self.b_stage, 4),
         ):
-            for x in range(4):
+            # two buffers: the buffer is an immediate offset; three: one address register per buffer and
+            # step (set up by the prologue), because the offsets no longer fit the 16-bit immediate
+            if self.stages == 2:
+                reg, boff = (vaddr + s if not tr else vaddr), buf * stage
+            else:
+                reg, boff = (vbuf + 4 * buf + s if not tr else vbuf + 4 * buf), 0
+            for x in range(nblk):
                 d = vbase + 4 * x
                 if not tr:
                     # address register per step; sub-tiles are 32 rows = 4096 bytes apart
-                    out.append("ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(vaddr + s), buf * stage + x * 4096))
+                    out.append("ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(reg), boff + x * 4096))
                 else:
-                    o = buf * stage + s * 8 * TR_BLOCK + x * 64
-                    out.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d, 2), vr(vaddr), o))
-                    out.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d + 2, 2), vr(vaddr), o + 512))
+                    o = boff + s * 8 * TR_BLOCK + x * 64
+                    out.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d, 2), vr(reg), o))
+                    out.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d + 2, 2), vr(reg), o + 512))
         return out
 
     def n_frag_reads(self):
@@ -142,7 +160,7 @@ class Variant:
     # -- MFMAs of one step on register set st
     def mfmas(self, st):
         out = []
-        for i in range(4):
+        for i in range(self.tm):
             for j in range(4):
                 a = vr(V_AF[st] + 4 * i, 4)
                 b = vr(V_BF[st] + 4 * j, 4)
@@ -156,8 +174,8 @@ class Variant:
     # s_ka / s_kb: SGPRs with the tile's byte offsets along K for A and B.  which: "head" or "loop".
     def dma(self, n, buf, which, s_tail, s_oob, s_ka, s_kb, tmp):
         out = []
-        is_a = n < 8
-        i = n if is_a else n - 8
+        is_a = n < self.na
+        i = n if is_a else n - self.na
         tr = self.a_tr if is_a else self.b_tr
         stage = self.a_stage if is_a else self.b_stage
         lbase = 0 if is_a else self.b_base
@@ -196,7 +214,9 @@ def fixup(e, v, which, buf):
         stage = v.a_stage if is_a else v.b_stage
         addr = V_FIX + (0 if is_a else 2) + which
         t = V_TMP + (0 if is_a else 4)
-        e("ds_read_b128 %s, %s offset:%d" % (vr(t, 4), vr(addr), buf * stage))
+        ta = V_TMP + 8 + (0 if is_a else 1)
+        e("v_add_u32 %s, %d, %s" % (vr(ta), buf * stage, vr(addr)))
+        e("ds_read_b128 %s, %s" % (vr(t, 4), vr(ta)))
     e("s_waitcnt lgkmcnt(0)")
     for is_a in (True, False):
         tr = v.a_tr if is_a else v.b_tr
@@ -205,9 +225,10 @@ def fixup(e, v, which, buf):
         stage = v.a_stage if is_a else v.b_stage
         addr = V_FIX + (0 if is_a else 2) + which
         t = V_TMP + (0 if is_a else 4)
+        ta = V_TMP + 8 + (0 if is_a else 1)
         for w in range(4):
             e("v_and_b32 %s, %s, %s" % (vr(t + w), sr(S_MASK + 4 * which + w), vr(t + w)))
-        e("ds_write_b128 %s, %s offset:%d" % (vr(addr), vr(t, 4), buf * stage))
+        e("ds_write_b128 %s, %s" % (vr(ta), vr(t, 4)))
 
 
 def interleave(e, mfmas, side_groups):
@@ -260,12 +281,12 @@ def gen_variant(v):
     e("s_sub_u32 %s, %s, 1" % (sr(s_last), sr(S_NK)))
     e("s_mov_b32 %s, 0" % sr(s_zero))
     # wave part of the LDS copy destinations: wave id is in s[S_SPARE]
-    e("s_mul_i32 %s, %s, %d" % (sr(s_waveA), sr(sT + 19), 8 * (TR_BLOCK if v.a_tr else 1024)))
+    e("s_mul_i32 %s, %s, %d" % (sr(s_waveA), sr(sT + 19), v.na * (TR_BLOCK if v.a_tr else 1024)))
     e("s_add_u32 %s, %s, %s" % (sr(s_waveA), sr(s_waveA), sr(S_LDS)))
     e("s_mul_i32 %s, %s, %d" % (sr(s_waveB), sr(sT + 19), 8 * (TR_BLOCK if v.b_tr else 1024)))
     e("s_add_u32 %s, %s, %s" % (sr(s_waveB), sr(s_waveB), sr(S_LDS)))
     # tile 0 -> buffer 0 (head offsets)
-    for n in range(16):
+    for n in range(v.ncopy):
         for ins in v.dma(n, 0, "head", 0, 0, s_zero, s_zero, V_TMP):
             e(ins)
     # tile 1 -> buffer 1, first 6 copies
@@ -273,12 +294,12 @@ def gen_variant(v):
     tile_masks(s_t1, s_tail1, s_oob1)
     e("s_mov_b32 %s, %s" % (sr(s_ka1), sr(S_ASTEP)))
     e("s_mov_b32 %s, %s" % (sr(s_kb1), sr(S_BSTEP)))
-    c3, c0, c1, c2 = COPY_SCHEDULE
+    c3, c0, c1, c2 = v.sched
     for n in range(c3):
         for ins in v.dma(n, 1, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)):
             e(ins)
     # zero the accumulators while the copies fly
-    for r in range(256):
+    for r in range(64 * v.tm):
         e("v_accvgpr_write_b32 a%d, 0" % r)
     e("s_waitcnt vmcnt(%d)" % c3)
     e("s_barrier")
@@ -335,7 +356,7 @@ def gen_variant(v):
         # step 2
         e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 3, 1)]
-        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, 16)]
+        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)]
         npf = 0
         if PREFETCH:
             e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), PREFETCH))
@@ -386,7 +407,7 @@ def gen_variant(v):
         # acc block (i, j), register 4 q + r  ->  C[m = 32 i + lane % 32][n = 32 j + 8 q + 4 (lane / 32) + r]
         t = V_TMP
         k = 0
-        for i in range(4):
+        for i in range(v.tm):
             for j in range(4):
                 for q in range(4):
                     b = t + 6 * (k % 4)
@@ -406,14 +427,15 @@ def gen_variant(v):
         voff, vrow, vsel = t + 16, t + 17, t + 18
         e("v_mov_b32 %s, %s" % (vr(voff), vr(V_EPI + 2)))
         e("v_mov_b32 %s, %s" % (vr(vrow), vr(V_EPI + 3)))
+        nrb = 8 * v.tm   # read-back instructions: 4 rows each
         for r in range(depth):
             e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r], 4), vr(V_EPI + 1), r * 4 * PITCH))
-        for r in range(32):
-            e("s_waitcnt lgkmcnt(%d)" % min(depth - 1, 31 - r))
+        for r in range(nrb):
+            e("s_waitcnt lgkmcnt(%d)" % min(depth - 1, nrb - 1 - r))
             e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
             e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vsel), vr(V_OOB), vr(voff)))
             e("buffer_store_dwordx4 %s, %s, %s, 0 offen" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
-            if r + depth < 32:
+            if r + depth < nrb:
                 # the store above must have read its data before the register is reloaded
                 e("s_nop 0")
                 e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r % depth], 4), vr(V_EPI + 1), (r + depth) * 4 * PITCH))
@@ -431,7 +453,7 @@ def gen_variant(v):
             e("s_mov_b64 %s, vcc" % sr(S_T + 24 + 2 * j, 2))
         k = 0
         e("s_mov_b32 %s, 0" % sr(S_T + 16))   # running row offset in bytes
-        for i in range(4):
+        for i in range(v.tm):
             for q in range(4):
                 for r in range(4):
                     row = 32 * i + 8 * q + r
@@ -469,13 +491,15 @@ def main():
     out.append("#define GMM_TILE_KC_STAGE %d" % KC_STAGE)
     out.append("#define GMM_TILE_TR_STAGE %d" % TR_STAGE)
     out.append("#define GMM_TILE_STAGING_BYTES %d" % STAGE_BYTES)
-    for a_tr in (0, 1):
-        for b_tr in (0, 1):
-            for f32 in (0, 1):
-                v = Variant(a_tr, b_tr, f32)
+    for a_tr, b_tr, f32, tm in [(a, b, f, t) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1)]:
+        if a_tr and tm != 4:
+            continue
+        if True:
+            if True:
+                v = Variant(a_tr, b_tr, f32, tm)
                 e = gen_variant(v)
                 out.append("")
-                out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32))
+                out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm))
                 out.append("  asm volatile(")
                 out.append(e.text())
                 out.append('      : "={s[92:99]}"(r.stamps)' if DBG_TIMING else "      :")

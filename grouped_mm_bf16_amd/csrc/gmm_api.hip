@@ -13,6 +13,8 @@ namespace {
 std::atomic<int> g_forced_path{GMM_PATH_AUTO};
 std::atomic<int> g_forced_config{-1};
 std::atomic<int> g_xcd_remap{1};
+std::atomic<int> g_forced_tall{-1};   // -1 auto, else 256 / 128
+std::atomic<int> g_forced_short{-1};  // -1 auto, 0 off, 64 on
 thread_local int t_last_path = 0;
 thread_local int t_last_config = -1;
 
@@ -107,6 +109,18 @@ int run(Problem& pr, hipStream_t stream) {
     int cfg = g_forced_config.load(std::memory_order_relaxed);
     if (cfg == GMM_CFG_ASM_256x256 && !can_asm) return GMM_ERR_UNSUPPORTED;
     if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = can_asm ? GMM_CFG_ASM_256x256 : GMM_CFG_REG_256x256;
+    // Tile heights of the assembly tile: 256-row tiles unless the launch would not even fill four rounds
+    // of the grid, then 128; 64-row tiles for group remainders whenever A is contiguous along K.
+    {
+      const int64_t tn = (p.N + 255) / 256;
+      int64_t est = (p.jag == GMM_JAG_M) ? (int64_t(p.M) / 256 + (p.G < p.M ? p.G : p.M)) * tn
+                                         : int64_t(p.G) * ((p.M + 255) / 256) * tn;
+      p.tall = (lay.a_kc && est < 4 * int64_t(cus)) ? 128 : 256;
+      p.shrt = lay.a_kc ? 64 : 0;
+      const int ft = g_forced_tall.load(std::memory_order_relaxed), fs = g_forced_short.load(std::memory_order_relaxed);
+      if (lay.a_kc && (ft == 256 || ft == 128)) p.tall = ft;
+      if (lay.a_kc && (fs == 0 || fs == 64)) p.shrt = fs;
+    }
     rc = gmm_launch_mfma(p, lay, pr.out_dtype, cfg, cus, stream);
     t_last_path = GMM_PATH_MFMA;
     t_last_config = cfg;
@@ -198,6 +212,11 @@ int gmm_last_path(void) { return t_last_path; }
 int gmm_set_mfma_config(int config) { return g_forced_config.exchange(config); }
 int gmm_last_mfma_config(void) { return t_last_config; }
 int gmm_set_xcd_remap(int on) { return g_xcd_remap.exchange(on ? 1 : 0); }
+int gmm_set_tile_heights(int tall, int shrt) {
+  g_forced_tall.store(tall);
+  g_forced_short.store(shrt);
+  return 0;
+}
 
 int64_t gmm_host_tile_list(const int32_t* offs_host, int32_t G, int32_t jagged, int32_t M, int32_t N, int32_t K,
                            int32_t tile_m, int32_t tile_n, int32_t align, int32_t xcd_remap,
@@ -229,6 +248,45 @@ int64_t gmm_host_tile_list(const int32_t* offs_host, int32_t G, int32_t jagged, 
       int32_t* r = records + int64_t(t) * 9;
       r[0] = tile.g; r[1] = tile.m0; r[2] = tile.n0; r[3] = tile.m_lo; r[4] = tile.m_hi;
       r[5] = tile.n_lo; r[6] = tile.n_hi; r[7] = tile.k_lo; r[8] = tile.k_hi;
+    }
+  }
+  return total;
+}
+
+int64_t gmm_host_tile_list2(const int32_t* offs_host, int32_t G, int32_t jagged, int32_t M, int32_t N, int32_t K,
+                            int32_t tall, int32_t shrt, int32_t tile_n, int32_t align, int32_t xcd_remap,
+                            int32_t num_workgroups, int32_t* records, int64_t capacity) {
+  if (G < 0 || jagged < 0 || jagged > 3 || jagged == GMM_JAG_N || tall <= 0 || shrt < 0 || tile_n <= 0 || align <= 0)
+    return -GMM_ERR_BAD_ARGUMENT;
+  if (jagged != GMM_JAG_NONE && (!offs_host || G < 1 || G >= GMM_MAX_GROUPS)) return -GMM_ERR_BAD_ARGUMENT;
+  if (xcd_remap && (num_workgroups <= 0 || num_workgroups % 8)) return -GMM_ERR_BAD_ARGUMENT;
+  GmmParams p{};
+  p.offs = offs_host;
+  p.G = G; p.jag = jagged; p.M = M; p.N = N; p.K = K; p.align = align; p.tall = tall; p.shrt = shrt;
+  const int extent = jagged == GMM_JAG_M ? M : K;
+  const int tn = gmm_cdiv(N, tile_n);
+  std::vector<int32_t> ct(size_t(G) + 1, 0), cs(size_t(G) + 1, 0);
+  for (int g = 0; g < G; ++g) {
+    int lo = 0, hi = 0, n_tall, n_short;
+    if (jagged != GMM_JAG_NONE) gmm_group_range(offs_host, g, extent, lo, hi);
+    gmm_split_rows(gmm_group_rows(jagged, lo, hi, M, align), tall, shrt, n_tall, n_short);
+    ct[g + 1] = ct[g] + n_tall * tn;
+    cs[g + 1] = cs[g] + n_short * tn;
+  }
+  const int total_tall = ct[G], total = ct[G] + cs[G];
+  for (int t = 0; t < total; ++t) {
+    const int tt = xcd_remap ? gmm_xcd_remap(t, total, num_workgroups) : t;
+    const int cls = tt < total_tall ? 0 : 1;
+    const int tc = cls ? tt - total_tall : tt;
+    const std::vector<int32_t>& cum = cls ? cs : ct;
+    const int g = gmm_find_group(cum.data(), G, tc);
+    int lo = 0, hi = 0;
+    if (jagged != GMM_JAG_NONE) gmm_group_range(offs_host, g, extent, lo, hi);
+    const GmmTile tile = gmm_make_tile2(p, g, lo, hi, cls, tc - cum[g], tile_n);
+    if (t < capacity && records) {
+      int32_t* r = records + int64_t(t) * 10;
+      r[0] = tile.g; r[1] = tile.m0; r[2] = tile.n0; r[3] = tile.m_lo; r[4] = tile.m_hi;
+      r[5] = tile.n_lo; r[6] = tile.n_hi; r[7] = tile.k_lo; r[8] = tile.k_hi; r[9] = tile.rows;
     }
   }
   return total;

@@ -90,6 +90,83 @@ __device__ __forceinline__ GmmTile gmm_locate_tile_divergent(const GmmParams& p,
   return gmm_make_tile(p, g, lo, hi, mt, nt, bm, bn);
 }
 
+// ---- two-height tile list (gmm_sched.h): tables cum[0] (tall) and cum[1] (short), each G + 1 entries ---- //
+template <int NT>
+__device__ __forceinline__ void gmm_scan_table(int32_t* cum) {
+  const int tid = threadIdx.x;
+  if (tid < 64) {
+    constexpr int PER = GMM_MAX_GROUPS / 64;
+    int v[PER];
+    int run = 0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) { run += cum[1 + tid * PER + i]; v[i] = run; }
+    int incl = run;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (tid >= d) incl += up;
+    }
+    const int before = incl - run;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) cum[1 + tid * PER + i] = v[i] + before;
+  }
+}
+
+// Returns the total number of tiles; total_tall gets the number of tall ones.
+template <int NT>
+__device__ __forceinline__ int gmm_build_tile_table2(const GmmParams& p, int bn, int32_t* cum_tall, int32_t* cum_short,
+                                                     int& total_tall) {
+  const int tid = threadIdx.x;
+  const int tn = gmm_cdiv(p.N, bn);
+  if (p.jag == GMM_JAG_NONE) {
+    int n_tall, n_short;
+    gmm_split_rows(p.M, p.tall, p.shrt, n_tall, n_short);
+    total_tall = p.G * n_tall * tn;
+    return total_tall + p.G * n_short * tn;
+  }
+  const int extent = p.jag == GMM_JAG_M ? p.M : p.K;
+  for (int g = tid; g < GMM_MAX_GROUPS; g += NT) {
+    int ct = 0, cs = 0;
+    if (g < p.G) {
+      int lo, hi, n_tall, n_short;
+      gmm_group_range(p.offs, g, extent, lo, hi);
+      gmm_split_rows(gmm_group_rows(p.jag, lo, hi, p.M, p.align), p.tall, p.shrt, n_tall, n_short);
+      ct = n_tall * tn;
+      cs = n_short * tn;
+    }
+    cum_tall[g + 1] = ct;
+    cum_short[g + 1] = cs;
+  }
+  if (tid == 0) { cum_tall[0] = 0; cum_short[0] = 0; }
+  __syncthreads();
+  gmm_scan_table<NT>(cum_tall);
+  gmm_scan_table<NT>(cum_short);
+  __syncthreads();
+  total_tall = cum_tall[p.G];
+  return total_tall + cum_short[p.G];
+}
+
+// Tile id -> tile, per lane (ids differ between lanes).
+__device__ __forceinline__ GmmTile gmm_locate_tile2(const GmmParams& p, const int32_t* cum_tall, const int32_t* cum_short,
+                                                    int total_tall, int t, int bn) {
+  const int cls = t < total_tall ? 0 : 1;
+  const int tc = cls ? t - total_tall : t;
+  int g, local, lo = 0, hi = 0;
+  if (p.jag == GMM_JAG_NONE) {
+    int n_tall, n_short;
+    gmm_split_rows(p.M, p.tall, p.shrt, n_tall, n_short);
+    const int per = (cls ? n_short : n_tall) * gmm_cdiv(p.N, bn);
+    g = tc / per;
+    local = tc - g * per;
+  } else {
+    const int32_t* cum = cls ? cum_short : cum_tall;
+    g = gmm_find_group(cum, p.G, tc);
+    local = tc - cum[g];
+    gmm_group_range(p.offs, g, p.jag == GMM_JAG_M ? p.M : p.K, lo, hi);
+  }
+  return gmm_make_tile2(p, g, lo, hi, cls, local, bn);
+}
+
 // ---- element types -------------------------------------------------------- //
 struct gmm_bf16 { uint16_t bits; };
 struct gmm_f16 { _Float16 v; };

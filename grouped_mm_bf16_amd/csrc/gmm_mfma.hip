@@ -261,17 +261,21 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) gmm_mfma_kernel(cons
 // Same tile list, but each tile's main loop and epilogue run as one hand-scheduled assembly block:
 // direct global -> LDS copies, no register staging, explicit registers.  A_TR / B_TR: the operand is
 // contiguous along M / N (not along K) and is read from LDS with transposing loads.
-template <int A_TR, int B_TR, int OUT_F32>
+// TALL_TM: height of the tall tiles in units of 64 rows (4 or 2); 64-row short tiles for group remainders
+// exist when A is contiguous along K (p.shrt == 64).
+template <int A_TR, int B_TR, int OUT_F32, int TALL_TM>
 __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[gmm_tile_lds_bytes<A_TR, B_TR>()];
-  __shared__ int32_t cum[GMM_MAX_GROUPS + 1];
+  __shared__ int32_t cum_tall[GMM_MAX_GROUPS + 1];
+  __shared__ int32_t cum_short[GMM_MAX_GROUPS + 1];
   __shared__ int32_t tiles[256][12];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
   constexpr int ESZ = OUT_F32 ? 4 : 2;
 
-  const int total = gmm_build_tile_table<256>(p, GMM_TILE_M, GMM_TILE_N, cum);
+  int total_tall;
+  const int total = gmm_build_tile_table2<256>(p, GMM_TILE_N, cum_tall, cum_short, total_tall);
   const uint16_t* __restrict__ A = static_cast<const uint16_t*>(p.a);
   const uint16_t* __restrict__ B = static_cast<const uint16_t*>(p.b);
   char* __restrict__ C = static_cast<char*>(p.c);
@@ -287,10 +291,10 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
     if (mine < total) {
       const int t = int(mine);
       const int tt = p.xcd_remap ? gmm_xcd_remap(t, total, gridDim.x) : t;
-      const GmmTile tile = gmm_locate_tile_divergent(p, cum, tt, GMM_TILE_M, GMM_TILE_N);
+      const GmmTile tile = gmm_locate_tile2(p, cum_tall, cum_short, total_tall, tt, GMM_TILE_N);
       int32_t* d = tiles[tid];
       d[0] = tile.g; d[1] = tile.m0; d[2] = tile.n0; d[3] = tile.m_lo; d[4] = tile.m_hi;
-      d[5] = tile.n_lo; d[6] = tile.n_hi; d[7] = tile.k_lo; d[8] = tile.k_hi;
+      d[5] = tile.n_lo; d[6] = tile.n_hi; d[7] = tile.k_lo; d[8] = tile.k_hi; d[9] = tile.rows;
     }
     __syncthreads();
     const int64_t left = (int64_t(total) - blockIdx.x + gridDim.x - 1) / gridDim.x - first;  // tiles of this workgroup from `first` on
@@ -302,6 +306,7 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       const int m_lo = __builtin_amdgcn_readfirstlane(d[3]), m_hi = __builtin_amdgcn_readfirstlane(d[4]);
       const int n_lo = __builtin_amdgcn_readfirstlane(d[5]), n_hi = __builtin_amdgcn_readfirstlane(d[6]);
       const int k_lo = __builtin_amdgcn_readfirstlane(d[7]), k_hi = __builtin_amdgcn_readfirstlane(d[8]);
+      const int rows = __builtin_amdgcn_readfirstlane(d[9]);
       // the copies move 16-byte chunks along K for an operand that is contiguous along K
       const int k_begin = (A_TR && B_TR) ? k_lo : (k_lo & ~7);
       const uint16_t* a = A + int64_t(g) * p.a_sg;
@@ -330,27 +335,33 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       dsc.klen = k_hi > k_lo ? k_hi - k_begin : 0;
       dsc.khead = k_lo - k_begin;
       dsc.row_rel0 = m0 - m_lo;
-      dsc.row_cnt = m_hi - m_lo;
+      // rows past the tile's own height belong to the next tile of the group
+      dsc.row_cnt = gmm_min(m_hi, m0 + rows) - m_lo;
       dsc.col_lo = gmm_max(n_lo - n0, 0);
       dsc.col_hi = gmm_min(n_hi - n0, GMM_TILE_N);
-      gmm_tile_compute<A_TR, B_TR, OUT_F32>(dsc, lds_base, lane, wave);
+      if constexpr (A_TR) {
+        gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane, wave);
+      } else {
+        if (rows == 64 * TALL_TM) gmm_tile_compute<A_TR, B_TR, OUT_F32, TALL_TM>(dsc, lds_base, lane, wave);
+        else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1>(dsc, lds_base, lane, wave);
+      }
     }
     if (left <= 256) break;
     __syncthreads();  // everyone is done with this batch of located tiles
   }
 }
 
-template <int OUT_F32>
+template <int OUT_F32, int TALL_TM>
 int launch_asm(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
   const dim3 grid(p.num_wg), block(256);
   if (lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32, TALL_TM>), grid, block, 0, stream, p);
   else if (lay.a_kc && !lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32, TALL_TM>), grid, block, 0, stream, p);
   else if (!lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32, 4>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32, 4>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 1;
 }
 
@@ -380,8 +391,11 @@ void gmm_mfma_tile_shape(int config, int& bm, int& bn) {
 int gmm_launch_mfma(GmmParams p, GmmLayout lay, int out_dtype, int config, int num_cus, hipStream_t stream) {
   p.num_wg = num_cus;
   if (config == GMM_CFG_ASM_256x256) {
-    if (out_dtype == GMM_DT_BF16) return launch_asm<0>(p, lay, stream);
-    if (out_dtype == GMM_DT_F32) return launch_asm<1>(p, lay, stream);
+    // a column-major A has only the 256-row tile
+    if (!lay.a_kc) { p.tall = 256; p.shrt = 0; }
+    if (p.tall != 128) p.tall = 256;
+    if (out_dtype == GMM_DT_BF16) return p.tall == 256 ? launch_asm<0, 4>(p, lay, stream) : launch_asm<0, 2>(p, lay, stream);
+    if (out_dtype == GMM_DT_F32) return p.tall == 256 ? launch_asm<1, 4>(p, lay, stream) : launch_asm<1, 2>(p, lay, stream);
     return -1;
   }
   if (out_dtype == GMM_DT_BF16) return launch_layout<256, 256, 2, 2, uint16_t>(p, lay, stream);

@@ -43,6 +43,8 @@ struct GmmParams {
   int64_t c_sg, c_sm, c_sn;
   int32_t xcd_remap;  // 1: renumber tiles so that each XCD works on a compact block
   int32_t num_wg;     // persistent grid size
+  int32_t tall;       // two-height tile list: rows of a "tall" tile (256 or 128) ...
+  int32_t shrt;       // ... and of a "short" tile for group remainders (64), or 0: tall tiles only
 };
 
 GMM_HD int gmm_cdiv(int a, int b) { return (a + b - 1) / b; }
@@ -112,6 +114,27 @@ GMM_HD int gmm_find_group(const int32_t* cum, int G, int t) {
   return lo;
 }
 
+// ---- two tile heights ------------------------------------------------------------------------ //
+// Skewed group sizes leave many groups far smaller than a tall tile.  The row range of a group is cut
+// into tall tiles; a remainder that fits one 64-row "short" tile becomes one (it streams B at the same
+// rate but wastes no MFMA work on rows that do not exist), a longer one pays for another tall tile: a
+// short tile runs at about half the speed per row, so two of them cost as much as a tall one.  All tall
+// tiles of all groups come first in the tile order, the short ones fill the tail of the launch.
+GMM_HD void gmm_split_rows(int rows, int tall, int shrt, int& n_tall, int& n_short) {
+  if (rows <= 0) { n_tall = 0; n_short = 0; return; }
+  if (shrt <= 0) { n_tall = gmm_cdiv(rows, tall); n_short = 0; return; }
+  n_tall = rows / tall;
+  const int rem = rows - n_tall * tall;
+  if (rem > shrt) { n_tall += 1; n_short = 0; }
+  else n_short = rem > 0 ? 1 : 0;
+}
+
+// Rows of group g that the tile grid has to span (from the aligned-down start when rows are jagged).
+GMM_HD int gmm_group_rows(int jag, int lo, int hi, int M, int align) {
+  if (jag != GMM_JAG_M) return M;
+  return hi > lo ? hi - (lo / align) * align : 0;
+}
+
 // One output tile, in global coordinates of the operands.
 struct GmmTile {
   int32_t g;
@@ -119,16 +142,40 @@ struct GmmTile {
   int32_t m_lo, m_hi;    // rows that may be stored: [m_lo, m_hi)
   int32_t n_lo, n_hi;    // columns that may be stored
   int32_t k_lo, k_hi;    // contraction range that contributes
+  int32_t rows;          // height of the tile (0: the kernel's only height)
 };
 
 GMM_HD GmmTile gmm_make_tile(const GmmParams& p, int g, int lo, int hi, int mt, int nt, int bm, int bn) {
   GmmTile t;
   t.g = g;
+  t.rows = 0;
   t.m0 = mt * bm; t.m_lo = 0; t.m_hi = p.M;
   t.n0 = nt * bn; t.n_lo = 0; t.n_hi = p.N;
   t.k_lo = 0; t.k_hi = p.K;
   if (p.jag == GMM_JAG_M) { t.m0 += (lo / p.align) * p.align; t.m_lo = lo; t.m_hi = hi; }
   if (p.jag == GMM_JAG_N) { t.n0 += (lo / p.align) * p.align; t.n_lo = lo; t.n_hi = hi; }
   if (p.jag == GMM_JAG_K) { t.k_lo = lo; t.k_hi = hi; }
+  return t;
+}
+
+// Tile of the two-height list: `cls` 0 = tall, 1 = short; `local` = index inside the group's tiles of
+// that class.  Not used with jagged columns.
+GMM_HD GmmTile gmm_make_tile2(const GmmParams& p, int g, int lo, int hi, int cls, int local, int bn) {
+  const int rows = gmm_group_rows(p.jag, lo, hi, p.M, p.align);
+  int n_tall, n_short;
+  gmm_split_rows(rows, p.tall, p.shrt, n_tall, n_short);
+  const int tn = gmm_cdiv(p.N, bn);
+  int mt, nt, m_off;
+  if (cls == 0) {
+    gmm_decode_in_group(local, n_tall, tn, mt, nt);
+    m_off = mt * p.tall;
+  } else {
+    mt = local % n_short;
+    nt = local / n_short;
+    m_off = n_tall * p.tall + mt * p.shrt;
+  }
+  GmmTile t = gmm_make_tile(p, g, lo, hi, 0, nt, p.tall, bn);
+  t.m0 += m_off;
+  t.rows = cls == 0 ? p.tall : p.shrt;
   return t;
 }

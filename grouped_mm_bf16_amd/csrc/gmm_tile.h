@@ -23,7 +23,8 @@ struct GmmTileRegs {
   gmm_v8i stamps;              // timing builds only: four 64-bit s_memrealtime stamps
 };
 
-template <int A_TR, int B_TR, int OUT_F32>
+// TM = MFMA block rows per wave: the tile is 64 * TM rows (256, 128 or 64) by 256 columns.
+template <int A_TR, int B_TR, int OUT_F32, int TM>
 __device__ __forceinline__ void gmm_tile_asm(GmmTileRegs& r);
 
 #include "gmm_tile_asm.inc"
@@ -72,14 +73,16 @@ struct GmmTileDesc {
   int col_lo, col_hi;    // columns [col_lo, col_hi) of the tile are stored (relative to n0)
 };
 
-template <int TR>
+// NI = copy instructions per wave and K tile for this operand (8 for 256 rows, 2 per 64 rows).
+template <int TR, int NI>
 __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int klen, int khead, int nk,
                                                  gmm_v8i& head, gmm_v8i& full, gmm_v8i& tail) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
+    if (i >= NI) { head[i] = full[i] = tail[i] = (int)GMM_OOB; continue; }
     int k, vo;
     if (!TR) {
-      const int row = wave * 64 + i * 8 + (lane >> 3);
+      const int row = wave * (NI * 8) + i * 8 + (lane >> 3);
       const int c = (lane & 7) ^ gmm_swz(row);
       k = c * 8;
       vo = row * ld * 2 + c * 16;
@@ -96,21 +99,23 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int
   }
 }
 
-template <int A_TR, int B_TR, int OUT_F32>
+template <int A_TR, int B_TR, int OUT_F32, int TM = 4>
 __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave,
                                                  gmm_v8i* stamps = nullptr) {
+  static_assert(TM == 4 || !A_TR, "short tiles exist for a K-contiguous A only");
+  constexpr int WROWS = 32 * TM;  // rows of the tile per wave row
   constexpr int A_STAGE = A_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE;
   const int wm = wave & 1, wn = wave >> 1;
   const int nk = (t.klen + GMM_TILE_K - 1) / GMM_TILE_K;
   GmmTileRegs r;
-  gmm_copy_offsets<A_TR>(lane, wave, t.a.ld, t.klen, t.khead, nk, r.voa_head, r.voa, r.voa_tail);
-  gmm_copy_offsets<B_TR>(lane, wave, t.b.ld, t.klen, t.khead, nk, r.vob_head, r.vob, r.vob_tail);
+  gmm_copy_offsets<A_TR, 2 * TM>(lane, wave, t.a.ld, t.klen, t.khead, nk, r.voa_head, r.voa, r.voa_tail);
+  gmm_copy_offsets<B_TR, 8>(lane, wave, t.b.ld, t.klen, t.khead, nk, r.vob_head, r.vob, r.vob_tail);
   const int q = lane >> 4, ii = lane & 15;
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
     const int chunk = 2 * s + (lane >> 5);
     if (!A_TR) {
-      const int row = wm * 128 + (lane & 31);
+      const int row = wm * WROWS + (lane & 31);
       r.ra_addr[s] = lds_base + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
     } else {
       r.ra_addr[s] = lds_base + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wm * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
@@ -127,14 +132,14 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   r.pf[1] = B_TR ? (wave * 16 + (lane >> 2)) * t.b.ld * 2 + (lane & 3) * 128 : (wave * 64 + lane) * t.b.ld * 2;
   int c_step, n_valid = 0;
   if (!OUT_F32) {
-    const int row_t = wm * 128 + (lane >> 4), col_t = wn * 128 + (lane & 15) * 8;
-    r.epi[0] = lds_base + wave * (128 * GMM_TILE_PITCH) + (lane & 31) * GMM_TILE_PITCH + 8 * (lane >> 5);
-    r.epi[1] = lds_base + wave * (128 * GMM_TILE_PITCH) + (lane >> 4) * GMM_TILE_PITCH + (lane & 15) * 16;
+    const int row_t = wm * WROWS + (lane >> 4), col_t = wn * 128 + (lane & 15) * 8;
+    r.epi[0] = lds_base + wave * (WROWS * GMM_TILE_PITCH) + (lane & 31) * GMM_TILE_PITCH + 8 * (lane >> 5);
+    r.epi[1] = lds_base + wave * (WROWS * GMM_TILE_PITCH) + (lane >> 4) * GMM_TILE_PITCH + (lane & 15) * 16;
     r.epi[2] = (col_t >= t.col_lo && col_t + 8 <= t.col_hi) ? (row_t * t.ldc + col_t) * 2 : (int)GMM_OOB;
     r.epi[3] = t.row_rel0 + row_t;
     c_step = 4 * t.ldc * 2;
   } else {
-    const int row_t = wm * 128 + 4 * (lane >> 5), col_t = wn * 128 + (lane & 31);
+    const int row_t = wm * WROWS + 4 * (lane >> 5), col_t = wn * 128 + (lane & 31);
     r.epi[0] = 0;
     r.epi[1] = lane & 31;
     r.epi[2] = (row_t * t.ldc + col_t) * 4;
@@ -153,12 +158,14 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   int flags = 0;
   if (!(A_TR && B_TR)) flags = (t.khead ? 1 : 0) | (ktail ? 2 : 0);
   {
-    const int row = threadIdx.x;                      // one row of each 256-row operand tile per thread
+    // one row of each operand tile per thread (A tiles shorter than 256 rows: several threads per row,
+    // all writing the same masked value)
+    const int row = threadIdx.x, row_a = threadIdx.x % (64 * TM);
     const int c_last = ((t.klen - 1) & (GMM_TILE_K - 1)) >> 3;
-    r.fix[0] = lds_base + row * 128 + ((0 ^ gmm_swz(row)) << 4);
-    r.fix[1] = lds_base + row * 128 + ((c_last ^ gmm_swz(row)) << 4);
-    r.fix[2] = r.fix[0] + 2 * A_STAGE;
-    r.fix[3] = r.fix[1] + 2 * A_STAGE;
+    r.fix[0] = lds_base + row_a * 128 + ((0 ^ gmm_swz(row_a)) << 4);
+    r.fix[1] = lds_base + row_a * 128 + ((c_last ^ gmm_swz(row_a)) << 4);
+    r.fix[2] = lds_base + 2 * A_STAGE + row * 128 + ((0 ^ gmm_swz(row)) << 4);
+    r.fix[3] = lds_base + 2 * A_STAGE + row * 128 + ((c_last ^ gmm_swz(row)) << 4);
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       const unsigned h0 = (2 * w >= t.khead) ? 0x0000ffffu : 0u, h1 = (2 * w + 1 >= t.khead) ? 0xffff0000u : 0u;
@@ -170,6 +177,6 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   const int sc[8] = {nk, a_step, b_step, (int)lds_base, t.row_cnt, c_step, n_valid, wave | (flags << 8)};
 #pragma unroll
   for (int i = 0; i < 8; ++i) r.scal[i] = __builtin_amdgcn_readfirstlane(sc[i]);
-  gmm_tile_asm<A_TR, B_TR, OUT_F32>(r);
+  gmm_tile_asm<A_TR, B_TR, OUT_F32, TM>(r);
   if (stamps) *stamps = r.stamps;
 }

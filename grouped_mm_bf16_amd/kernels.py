@@ -124,6 +124,17 @@ def forced_mfma_config(config: int):
         lib.gmm_set_mfma_config(prev)
 
 
+@contextlib.contextmanager
+def forced_tile_heights(tall: int, shrt: int):
+    """Force the tile heights of the assembly tile (tall 256 / 128, short 64 / 0; -1 = automatic)."""
+    lib = _lib.load()
+    lib.gmm_set_tile_heights(tall, shrt)
+    try:
+        yield
+    finally:
+        lib.gmm_set_tile_heights(-1, -1)
+
+
 def last_path() -> str:
     """Kernel family used by this thread's last launch: "generic", "mfma" or "none"."""
     return {0: "none", _lib.PATH_GENERIC: "generic", _lib.PATH_MFMA: "mfma"}[_lib.load().gmm_last_path()]

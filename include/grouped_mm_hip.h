@@ -99,6 +99,9 @@ int gmm_set_mfma_config(int config);
 int gmm_last_mfma_config(void);
 /* 0 / 1: renumber tiles per XCD (default 1). */
 int gmm_set_xcd_remap(int on);
+/* Tile heights of the assembly tile: tall = 256 or 128 (-1: chosen from the shapes), shrt = 64 or 0
+ * (-1: 64 whenever the first operand is contiguous along the contraction). */
+int gmm_set_tile_heights(int tall, int shrt);
 
 /* Host-side run of the tile scheduler that the kernels execute on the device:
  * writes up to `capacity` records of 9 int32 (group, m0, n0, m_lo, m_hi, n_lo,
@@ -110,6 +113,14 @@ int64_t gmm_host_tile_list(const int32_t* offs_host, int32_t G, int32_t jagged,
                            int32_t tile_m, int32_t tile_n, int32_t align,
                            int32_t xcd_remap, int32_t num_workgroups,
                            int32_t* records, int64_t capacity);
+
+/* Same for the two-height tile list of the assembly tile (tall tiles first, then 64-row tiles for group
+ * remainders): records of 10 int32, the tenth being the tile's height.  jagged: 0, 1 or 3. */
+int64_t gmm_host_tile_list2(const int32_t* offs_host, int32_t G, int32_t jagged,
+                            int32_t M, int32_t N, int32_t K,
+                            int32_t tall, int32_t shrt, int32_t tile_n, int32_t align,
+                            int32_t xcd_remap, int32_t num_workgroups,
+                            int32_t* records, int64_t capacity);
 
 #ifdef __cplusplus
 }

@@ -131,3 +131,73 @@ def test_random_lists_exact_cover():
         align = int(rng.choice([1, 8]))
         rec = tile_list(sizes, ROWS, sum(sizes), 40, 8, bm, 32, align, remap=int(rng.integers(0, 2)), num_wg=16)
         assert (coverage(rec, G, sum(sizes), 40, bm, 32, False) == 1).all()
+
+
+# ---------------------------------------------------------------- two tile heights (assembly tile)
+def tile_list2(sizes, jag, M, N, K, tall, shrt, align=1, remap=0, num_wg=256):
+    lib = _lib.load()
+    offs = np.cumsum(sizes).astype(np.int32) if jag != NONE else np.zeros(1, np.int32)
+    G = len(sizes)
+    n = lib.gmm_host_tile_list2(offs.ctypes.data, G, jag, M, N, K, tall, shrt, 256, align, remap, num_wg, None, 0)
+    assert n >= 0
+    rec = np.zeros((max(n, 1), 10), np.int32)
+    assert lib.gmm_host_tile_list2(offs.ctypes.data, G, jag, M, N, K, tall, shrt, 256, align, remap, num_wg,
+                                   rec.ctypes.data, n) == n
+    return rec[:n]
+
+
+def coverage2(rec, G, M, N, per_group_out):
+    cnt = np.zeros((G if per_group_out else 1, M, N), np.int32)
+    for g, m0, n0, m_lo, m_hi, n_lo, n_hi, _, _, rows in rec:
+        r0, r1 = max(m0, m_lo), min(m0 + rows, m_hi)
+        c0, c1 = max(n0, n_lo), min(n0 + 256, n_hi)
+        assert r1 > r0 and c1 > c0, "a tile that stores nothing"
+        cnt[g if per_group_out else 0, r0:r1, c0:c1] += 1
+    return cnt
+
+
+@pytest.mark.parametrize("sizes", SIZE_LISTS + [[4812, 1663, 1610, 1663, 1656, 1682, 1633, 1665], [129, 128, 127, 65, 64, 63, 1]])
+@pytest.mark.parametrize("tall,shrt,align", [(256, 64, 1), (128, 64, 1), (256, 0, 1), (256, 0, 8), (256, 64, 8)])
+def test_two_heights_jagged_rows_exact_cover(sizes, tall, shrt, align):
+    M, N = sum(sizes), 300
+    if M == 0:
+        return
+    rec = tile_list2(sizes, ROWS, M, N, 16, tall, shrt, align, remap=1, num_wg=16)
+    assert (coverage2(rec, len(sizes), M, N, False) == 1).all()
+    heights = set(int(r[9]) for r in rec)
+    assert heights <= {tall, shrt}
+    # tall tiles come first in the launch order when ids are not renumbered
+    plain = tile_list2(sizes, ROWS, M, N, 16, tall, shrt, align)
+    hs = [int(r[9]) for r in plain]
+    assert hs == sorted(hs, reverse=True)
+    # a remainder that fits one short tile never pays for a tall tile
+    if shrt and align == 1:
+        for g, sz in enumerate(sizes):
+            rem = sz % tall
+            mine = [r for r in plain if r[0] == g and r[2] == 0]
+            if 0 < rem <= shrt:
+                assert sum(1 for r in mine if r[9] == shrt) == 1
+            else:
+                assert all(r[9] == tall for r in mine)
+
+
+@pytest.mark.parametrize("tall,shrt", [(256, 64), (128, 64), (256, 0)])
+def test_two_heights_contraction_and_batched(tall, shrt):
+    sizes = [7, 0, 1, 13, 11]
+    rec = tile_list2(sizes, CONTRACTION, 330, 300, sum(sizes), tall, shrt)
+    assert (coverage2(rec, 5, 330, 300, True) == 1).all()  # also the empty group
+    offs = np.cumsum(sizes)
+    for r in rec:
+        assert r[7] == offs[r[0]] - sizes[r[0]] and r[8] == offs[r[0]]
+    rec = tile_list2([0] * 5, NONE, 330, 300, 16, tall, shrt)
+    assert (coverage2(rec, 5, 330, 300, True) == 1).all()
+
+
+def test_two_heights_fine_grained_fixture(golden_dir):
+    import json, os
+    with open(os.path.join(golden_dir, "group_sizes.json")) as f:
+        sizes = json.load(f)["fine_grained_top8_g128"]
+    rec = tile_list2(sizes, ROWS, 32768, 768, 2048, 128, 64, remap=1, num_wg=256)
+    assert (coverage2(rec, 128, 32768, 768, False) == 1).all()
+    rows_paid = sum(int(r[9]) for r in rec if r[2] == 0)
+    assert rows_paid < 1.2 * 32768  # 256-row tiles alone pay for 54784 rows here
