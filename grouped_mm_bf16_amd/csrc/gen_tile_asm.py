@@ -74,7 +74,7 @@ V_EPI = 184            # 184: stage write addr, 185: stage read addr, 186: store
 V_OOB = 188            # constant 0x80000000
 V_PF = 192             # 192: A prefetch offset, 193: B prefetch offset
 V_PFD = 96             # dummy destinations of the prefetch loads (96, 97)
-STAGES_SHORT = int(os.environ.get('GMM_GEN_STAGES_SHORT', '2'))  # LDS buffers of the 128- and 64-row tiles
+STAGES_SHORT = int(os.environ.get('GMM_GEN_STAGES_SHORT', '3'))  # LDS buffers of the 128- and 64-row tiles
 V_BUFA, V_BUFB = 98, 110  # three-buffer variants: fragment addresses per (buffer, step), 12 + 12 registers
 V_FIX = 196            # 196: A first-chunk addr, 197: A last-chunk addr, 198 / 199: same for B (buffer 0)
 S_MASK = 28            # s[28:31] keep-mask of the first chunk of the k range, s[32:35] of the last chunk
@@ -289,19 +289,32 @@ def gen_variant(v):
     for n in range(v.ncopy):
         for ins in v.dma(n, 0, "head", 0, 0, s_zero, s_zero, V_TMP):
             e(ins)
-    # tile 1 -> buffer 1, first 6 copies
-    e("s_mov_b32 %s, 1" % sr(s_t1))
-    tile_masks(s_t1, s_tail1, s_oob1)
-    e("s_mov_b32 %s, %s" % (sr(s_ka1), sr(S_ASTEP)))
-    e("s_mov_b32 %s, %s" % (sr(s_kb1), sr(S_BSTEP)))
+    S = v.stages
     c3, c0, c1, c2 = v.sched
-    for n in range(c3):
-        for ins in v.dma(n, 1, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)):
-            e(ins)
+    if S == 3:
+        # fragment read addresses per buffer (the wrapper passes those of buffer 0)
+        for is_a in (True, False):
+            tr = v.a_tr if is_a else v.b_tr
+            stage = v.a_stage if is_a else v.b_stage
+            src, dst = (V_RA, V_BUFA) if is_a else (V_RB, V_BUFB)
+            for buf in range(S):
+                for st in range(1 if tr else 4):
+                    e("v_add_u32 %s, %d, %s" % (vr(dst + 4 * buf + st), buf * stage, vr(src + st)))
+    # tiles 1 .. S - 2 -> their buffers in full, tile S - 1 -> buffer S - 1: the first c3 copies
+    slots = [(s_tail1, s_oob1, s_ka1, s_kb1), (s_tail2, s_oob2, s_ka2, s_kb2)]
+    for tix in range(1, S):
+        s_tail, s_oob, s_ka, s_kb = slots[tix - 1]
+        e("s_mov_b32 %s, %d" % (sr(s_t1), tix))
+        tile_masks(s_t1, s_tail, s_oob)
+        e("s_mul_i32 %s, %s, %d" % (sr(s_ka), sr(S_ASTEP), tix))
+        e("s_mul_i32 %s, %s, %d" % (sr(s_kb), sr(S_BSTEP), tix))
+        for n in range(v.ncopy if tix < S - 1 else c3):
+            for ins in v.dma(n, tix, "loop", s_tail, s_oob, s_ka, s_kb, V_TMP + (n % 8)):
+                e(ins)
     # zero the accumulators while the copies fly
     for r in range(64 * v.tm):
         e("v_accvgpr_write_b32 a%d, 0" % r)
-    e("s_waitcnt vmcnt(%d)" % c3)
+    e("s_waitcnt vmcnt(%d)" % ((S - 2) * v.ncopy + c3))
     e("s_barrier")
     stamp(1)
     has_kc = not (v.a_tr and v.b_tr)
@@ -333,30 +346,31 @@ def gen_variant(v):
     def ktile(buf):
         # on entry: fragments of step 0 in set 0 (in flight); copies 0..5 of tile kt+1 in flight
         e("; ---- k tile on buffer %d" % buf)
-        # K offsets and masks of tiles kt+1 and kt+2
-        e("s_add_u32 %s, %s, 1" % (sr(s_t1), sr(s_kt)))
+        # K offsets and masks of tiles kt + S - 1 (copied during steps 0..2) and kt + S (step 3)
+        e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), S - 1))
         tile_masks(s_t1, s_tail1, s_oob1)
         e("s_mul_i32 %s, %s, %s" % (sr(s_ka1), sr(s_t1), sr(S_ASTEP)))
         e("s_mul_i32 %s, %s, %s" % (sr(s_kb1), sr(s_t1), sr(S_BSTEP)))
-        e("s_add_u32 %s, %s, 2" % (sr(s_t1), sr(s_kt)))
+        e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), S))
         tile_masks(s_t1, s_tail2, s_oob2)
         e("s_mul_i32 %s, %s, %s" % (sr(s_ka2), sr(s_t1), sr(S_ASTEP)))
         e("s_mul_i32 %s, %s, %s" % (sr(s_kb2), sr(s_t1), sr(S_BSTEP)))
-        nb = buf ^ 1
-        # step 0: MFMA set 0, read step 1 -> set 1, copies 6..10 of tile kt+1 -> other buffer
+        nb = (buf + 1) % S       # buffer of tile kt + 1
+        cb = (buf + S - 1) % S   # buffer of tile kt + S - 1
+        # step 0: MFMA set 0, read step 1 -> set 1, next copies of tile kt + S - 1
         e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 1, 1)]
-        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)]
+        side += [v.dma(n, cb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)]
         interleave(e, v.mfmas(0), side)
         # step 1
         e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 2, 0)]
-        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)]
+        side += [v.dma(n, cb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)]
         interleave(e, v.mfmas(1), side)
         # step 2
         e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 3, 1)]
-        side += [v.dma(n, nb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)]
+        side += [v.dma(n, cb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)]
         npf = 0
         if PREFETCH:
             e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), PREFETCH))
@@ -367,7 +381,7 @@ def gen_variant(v):
             npf = 2
         interleave(e, v.mfmas(0), side)
         # tile kt+1 has landed for this wave; after the barrier for all, and `buf` is free
-        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % npf)
+        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % ((S - 2) * v.ncopy + npf))
         if not DBG_NO_BARRIER:
             e("s_barrier")
         if not (v.a_tr and v.b_tr):
@@ -381,17 +395,18 @@ def gen_variant(v):
             e("s_waitcnt lgkmcnt(0)")
             e("s_barrier")
             e.label("L_nofix%d_%s" % (buf + 1, L))
-        # step 3: MFMA set 1, read step 0 of the next tile -> set 0, copies 0..5 of tile kt+2 -> buf
+        # step 3: MFMA set 1, read step 0 of the next tile -> set 0, first copies of tile kt + S -> buf
         side = [[x] for x in v.frag_reads(nb, 0, 0)]
         side += [v.dma(n, buf, "loop", s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, c3)]
         interleave(e, v.mfmas(1), side)
         e("s_add_u32 %s, %s, 1" % (sr(s_kt), sr(s_kt)))
 
     e.label("L_loop_%s" % L)
-    ktile(0)
-    e("s_cmp_ge_u32 %s, %s" % (sr(s_kt), sr(S_NK)))
-    e("s_cbranch_scc1 L_done_%s" % L)
-    ktile(1)
+    for buf in range(S - 1):
+        ktile(buf)
+        e("s_cmp_ge_u32 %s, %s" % (sr(s_kt), sr(S_NK)))
+        e("s_cbranch_scc1 L_done_%s" % L)
+    ktile(S - 1)
     e("s_cmp_lt_u32 %s, %s" % (sr(s_kt), sr(S_NK)))
     e("s_cbranch_scc1 L_loop_%s" % L)
     e.label("L_done_%s" % L)
@@ -476,7 +491,7 @@ def gen_variant(v):
 
 def clobbers():
     c = ["memory", "vcc", "scc"]
-    c += ["v%d" % i for i in range(0, 98)] + ["v%d" % V_OOB]
+    c += ["v%d" % i for i in range(0, 122)] + ["v%d" % V_OOB]
     c += ["a%d" % i for i in range(256)]
     c += ["s%d" % i for i in range(S_T, S_T + 34)]
     return ", ".join('"%s"' % x for x in c)
@@ -491,6 +506,7 @@ def main():
     out.append("#define GMM_TILE_KC_STAGE %d" % KC_STAGE)
     out.append("#define GMM_TILE_TR_STAGE %d" % TR_STAGE)
     out.append("#define GMM_TILE_STAGING_BYTES %d" % STAGE_BYTES)
+    out.append("#define GMM_TILE_STAGES_SHORT %d" % STAGES_SHORT)
     for a_tr, b_tr, f32, tm in [(a, b, f, t) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1)]:
         if a_tr and tm != 4:
             continue

@@ -265,10 +265,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) gmm_mfma_kernel(cons
 // exist when A is contiguous along K (p.shrt == 64).
 template <int A_TR, int B_TR, int OUT_F32, int TALL_TM>
 __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
-  __shared__ __attribute__((aligned(1024))) char lds[gmm_tile_lds_bytes<A_TR, B_TR>()];
+  constexpr int LDS_TALL = gmm_tile_lds_bytes<A_TR, B_TR, TALL_TM>();
+  constexpr int LDS_SHORT = A_TR ? 0 : gmm_tile_lds_bytes<0, B_TR, 1>();
+  constexpr int BATCH = 32;  // tiles located at a time
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_TALL > LDS_SHORT ? LDS_TALL : LDS_SHORT];
   __shared__ int32_t cum_tall[GMM_MAX_GROUPS + 1];
   __shared__ int32_t cum_short[GMM_MAX_GROUPS + 1];
-  __shared__ int32_t tiles[256][12];
+  __shared__ int32_t tiles[BATCH][10];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
@@ -284,11 +287,11 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
   const int ldc = int(p.c_sm);
 
   // This workgroup's tiles are blockIdx.x, blockIdx.x + gridDim.x, ...  Locating a tile (binary search
-  // over the groups, reads of offs, integer divisions) costs microseconds, so the 256 threads locate
-  // the next 256 tiles of the workgroup at once and leave them in LDS for the tile loop to pick up.
-  for (int first = 0;; first += 256) {
+  // over the groups, reads of offs, integer divisions) costs microseconds, so BATCH threads locate the
+  // next BATCH tiles of the workgroup at once and leave them in LDS for the tile loop to pick up.
+  for (int first = 0;; first += BATCH) {
     const int64_t mine = int64_t(blockIdx.x) + int64_t(first + tid) * gridDim.x;
-    if (mine < total) {
+    if (tid < BATCH && mine < total) {
       const int t = int(mine);
       const int tt = p.xcd_remap ? gmm_xcd_remap(t, total, gridDim.x) : t;
       const GmmTile tile = gmm_locate_tile2(p, cum_tall, cum_short, total_tall, tt, GMM_TILE_N);
@@ -298,7 +301,7 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
     }
     __syncthreads();
     const int64_t left = (int64_t(total) - blockIdx.x + gridDim.x - 1) / gridDim.x - first;  // tiles of this workgroup from `first` on
-    const int here = left < 256 ? int(left) : 256;
+    const int here = left < BATCH ? int(left) : BATCH;
     for (int j = 0; j < here; ++j) {
       const int32_t* d = tiles[j];
       const int g = __builtin_amdgcn_readfirstlane(d[0]);
@@ -346,7 +349,7 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
         else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1>(dsc, lds_base, lane, wave);
       }
     }
-    if (left <= 256) break;
+    if (left <= BATCH) break;
     __syncthreads();  // everyone is done with this batch of located tiles
   }
 }

@@ -32,11 +32,24 @@ __device__ __forceinline__ void gmm_tile_asm(GmmTileRegs& r);
 constexpr int GMM_TILE_M = 256, GMM_TILE_N = 256, GMM_TILE_K = 64;
 constexpr unsigned GMM_OOB = 0x80000000u;
 
-// LDS bytes one workgroup needs for a layout pair (pipeline buffers or the bf16 staging area).
-template <int A_TR, int B_TR>
+// Pipeline depth and LDS layout of a tile of 64 * TM rows: `stages` buffers of A from offset 0, then as
+// many of B.  The 256-row tile has two buffers (LDS is full); the shorter ones have
+// GMM_TILE_STAGES_SHORT, and with three their A buffers shrink to the rows they hold.
+template <int A_TR, int TM>
+struct GmmTileLayout {
+  static constexpr int stages = TM == 4 ? 2 : GMM_TILE_STAGES_SHORT;
+  static constexpr int a_stage = A_TR ? GMM_TILE_TR_STAGE : (stages == 3 ? 64 * TM * 128 : GMM_TILE_KC_STAGE);
+  static constexpr int b_base = stages * a_stage;
+};
+
+// LDS bytes one workgroup needs for tiles of 64 * TM rows: the pipeline buffers, or the staging area of
+// the bf16 epilogue (one padded row of 256 columns per tile row).
+template <int A_TR, int B_TR, int TM>
 constexpr int gmm_tile_lds_bytes() {
-  constexpr int pipe = 2 * (A_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE) + 2 * (B_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE);
-  return pipe > GMM_TILE_STAGING_BYTES ? pipe : GMM_TILE_STAGING_BYTES;
+  using L = GmmTileLayout<A_TR, TM>;
+  constexpr int pipe = L::b_base + L::stages * (B_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE);
+  constexpr int staging = 64 * TM * 2 * GMM_TILE_PITCH;
+  return pipe > staging ? pipe : staging;
 }
 
 __device__ __forceinline__ gmm_v4i gmm_make_rsrc(const void* p, long long bytes) {
@@ -104,7 +117,7 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
                                                  gmm_v8i* stamps = nullptr) {
   static_assert(TM == 4 || !A_TR, "short tiles exist for a K-contiguous A only");
   constexpr int WROWS = 32 * TM;  // rows of the tile per wave row
-  constexpr int A_STAGE = A_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE;
+  constexpr int B_BASE = GmmTileLayout<A_TR, TM>::b_base;
   const int wm = wave & 1, wn = wave >> 1;
   const int nk = (t.klen + GMM_TILE_K - 1) / GMM_TILE_K;
   GmmTileRegs r;
@@ -122,9 +135,9 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
     }
     if (!B_TR) {
       const int row = wn * 128 + (lane & 31);
-      r.rb_addr[s] = lds_base + 2 * A_STAGE + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
+      r.rb_addr[s] = lds_base + B_BASE + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
     } else {
-      r.rb_addr[s] = lds_base + 2 * A_STAGE + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wn * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
+      r.rb_addr[s] = lds_base + B_BASE + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wn * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
     }
   }
   // L2 prefetch: 256 cache lines per operand and K tile, one per lane
@@ -164,8 +177,8 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
     const int c_last = ((t.klen - 1) & (GMM_TILE_K - 1)) >> 3;
     r.fix[0] = lds_base + row_a * 128 + ((0 ^ gmm_swz(row_a)) << 4);
     r.fix[1] = lds_base + row_a * 128 + ((c_last ^ gmm_swz(row_a)) << 4);
-    r.fix[2] = lds_base + 2 * A_STAGE + row * 128 + ((0 ^ gmm_swz(row)) << 4);
-    r.fix[3] = lds_base + 2 * A_STAGE + row * 128 + ((c_last ^ gmm_swz(row)) << 4);
+    r.fix[2] = lds_base + B_BASE + row * 128 + ((0 ^ gmm_swz(row)) << 4);
+    r.fix[3] = lds_base + B_BASE + row * 128 + ((c_last ^ gmm_swz(row)) << 4);
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       const unsigned h0 = (2 * w >= t.khead) ? 0x0000ffffu : 0u, h1 = (2 * w + 1 >= t.khead) ? 0xffff0000u : 0u;
