@@ -45,6 +45,8 @@ import sys
 # of the next K tile; the tile must have landed at that tile's barrier (end of its step 2).
 COPY_SCHEDULE = tuple(int(x) for x in os.environ.get("GMM_GEN_COPY_SCHEDULE", "8,8,0,0").split(","))
 assert len(COPY_SCHEDULE) == 4 and sum(COPY_SCHEDULE) == 16
+COPY_SCHEDULE8 = tuple(int(x) for x in os.environ.get("GMM_GEN_COPY_SCHEDULE8", "4,4,0,0").split(","))  # 8 waves: 8 copies
+assert len(COPY_SCHEDULE8) == 4 and sum(COPY_SCHEDULE8) == 8
 
 # L2 prefetch distance in K tiles (0 = off): in step 2 of K tile kt every lane touches one cache line of
 # K tile kt + PREFETCH of each operand, so that the copies issued two tiles later hit in L2.
@@ -53,7 +55,10 @@ PREFETCH = int(os.environ.get("GMM_GEN_PREFETCH", "0"))
 # timing experiments only (results are wrong with these on)
 DBG_NO_COPY = int(os.environ.get("GMM_GEN_DBG_NO_COPY", "0"))
 DBG_NO_BARRIER = int(os.environ.get("GMM_GEN_DBG_NO_BARRIER", "0"))
+DBG_COPY_OOB = int(os.environ.get("GMM_GEN_DBG_COPY_OOB", "0"))  # timing only: loop copies fetch nothing (write zeros)
+DBG_NO_READS = int(os.environ.get("GMM_GEN_DBG_NO_READS", "0"))  # timing only: no fragment reads in the loop
 DBG_NO_MASK = int(os.environ.get("GMM_GEN_DBG_NO_MASK", "0"))
+DBG_VMCNT = int(os.environ.get("GMM_GEN_DBG_VMCNT", "-1"))  # timing experiments only: copies left in flight at the K-tile barrier
 DBG_TIMING = int(os.environ.get("GMM_GEN_DBG_TIMING", "0"))  # phase timestamps in s[92:99] (extra asm output)
 
 PITCH = 272           # bytes per staged row of 128 bf16 (256 + 16: shifts banks per row)
@@ -62,21 +67,38 @@ KC_STAGE = 256 * 64 * 2
 TR_STAGE = 32 * TR_BLOCK
 STAGE_BYTES = 4 * 128 * PITCH
 
-# ---- fixed register map ----------------------------------------------------
-V_AF = [0, 16]        # A fragment sets (4 x 4 registers each)
-V_BF = [32, 48]
-V_TMP = 64            # 64..95
-V_VOA_HEAD, V_VOB_HEAD = 128, 136
-V_VOA, V_VOB = 144, 152
-V_VOA_TAIL, V_VOB_TAIL = 160, 168
-V_RA, V_RB = 176, 180  # fragment read addresses (4 + 4)
-V_EPI = 184            # 184: stage write addr, 185: stage read addr, 186: store voffset, 187: row - row_lo
-V_OOB = 188            # constant 0x80000000
-V_PF = 192             # 192: A prefetch offset, 193: B prefetch offset
-V_PFD = 96             # dummy destinations of the prefetch loads (96, 97)
+# ---- fixed register maps ---------------------------------------------------
+# 4 waves (one per SIMD, 128 x 128 per wave, 256 accumulators): the wave owns all 512 registers of a lane.
+# 8 waves (two per SIMD, 128 x 64 per wave, 128 accumulators): 128 + 128 registers per wave.
 STAGES_SHORT = int(os.environ.get('GMM_GEN_STAGES_SHORT', '3'))  # LDS buffers of the 128- and 64-row tiles
-V_BUFA, V_BUFB = 98, 110  # three-buffer variants: fragment addresses per (buffer, step), 12 + 12 registers
-V_FIX = 196            # 196: A first-chunk addr, 197: A last-chunk addr, 198 / 199: same for B (buffer 0)
+REGMAPS = {
+    4: dict(V_AF=[0, 16],        # A fragment sets (4 x 4 registers each)
+            V_BF=[32, 48],
+            V_TMP=64,            # 64..95
+            V_VOA_HEAD=128, V_VOB_HEAD=136, V_VOA=144, V_VOB=152, V_VOA_TAIL=160, V_VOB_TAIL=168,
+            V_RA=176, V_RB=180,  # fragment read addresses (4 + 4)
+            V_EPI=184,           # +0: stage write addr, +1: stage read addr, +2: store voffset, +3: row - row_lo
+            V_OOB=188,           # constant 0x80000000
+            V_PF=192,            # A / B prefetch offsets
+            V_PFD=96,            # dummy destinations of the prefetch loads (96, 97)
+            V_BUFA=98, V_BUFB=110,  # three-buffer variants: fragment addresses per (buffer, step), 12 + 12
+            V_FIX=196,           # A first-chunk addr, A last-chunk addr, same for B (buffer 0)
+            V_CLOBBER=122),
+    8: dict(V_AF=[0, 24],        # A 4 x 4 registers, B 2 x 4 registers per set
+            V_BF=[16, 40],
+            V_TMP=48,            # 48..79
+            V_VOA_HEAD=80, V_VOB_HEAD=84, V_VOA=88, V_VOB=92, V_VOA_TAIL=96, V_VOB_TAIL=100,
+            V_RA=104, V_RB=108, V_EPI=112, V_FIX=116, V_OOB=120,
+            V_PF=None, V_PFD=None, V_BUFA=None, V_BUFB=None,
+            V_CLOBBER=80),
+}
+
+
+def use_regmap(waves):
+    globals().update(REGMAPS[waves])
+
+
+use_regmap(4)
 S_MASK = 28            # s[28:31] keep-mask of the first chunk of the k range, s[32:35] of the last chunk
 
 S_RA, S_RB, S_RC = 36, 40, 44   # buffer resources
@@ -99,8 +121,7 @@ class Emit:
         return "\n".join('      "%s\\n\\t"' % l for l in self.lines)
 
 
-def acc(i, j):
-    return (4 * i + j) * 16
+PITCH8 = 144          # 8 waves: bytes per staged row of 64 bf16 (128 + 16)
 
 
 def vr(base, n=1):
@@ -114,13 +135,15 @@ def sr(base, n=1):
 class Variant:
     """tm = MFMA block rows per wave: the tile is 64 tm rows (256 / 128 / 64) by 256 columns."""
 
-    def __init__(self, a_tr, b_tr, out_f32, tm=4):
-        self.a_tr, self.b_tr, self.out_f32, self.tm = a_tr, b_tr, out_f32, tm
-        assert tm in (1, 2, 4) and (tm == 4 or not a_tr)
-        self.na = 2 * tm                 # copies of the A tile per wave and K tile (B: always 8)
-        self.ncopy = self.na + 8
-        c3 = (self.ncopy + 1) // 2 if COPY_SCHEDULE == (8, 8, 0, 0) else None
-        self.sched = (c3, self.ncopy - c3, 0, 0) if c3 is not None else COPY_SCHEDULE
+    def __init__(self, a_tr, b_tr, out_f32, tm=4, waves=4):
+        self.a_tr, self.b_tr, self.out_f32, self.tm, self.waves = a_tr, b_tr, out_f32, tm, waves
+        assert tm in (1, 2, 4) and (tm == 4 or not a_tr) and (waves == 4 or (waves == 8 and tm == 4 and not PREFETCH))
+        self.tn = 16 // waves            # 32-column MFMA blocks per wave (the wave grid is 2 x waves / 2)
+        self.na = 8 * tm // waves        # copies of the A tile per wave and K tile
+        self.nb = 32 // waves            # ... of the B tile
+        self.ncopy = self.na + self.nb
+        c3 = (self.ncopy + 1) // 2
+        self.sched = COPY_SCHEDULE if (tm == 4 and waves == 4) else COPY_SCHEDULE8 if waves == 8 else (c3, self.ncopy - c3, 0, 0)
         # LDS buffers per operand: 2 for the 256-row tile (LDS is full), 3 for the shorter ones, whose K
         # tiles are short of MFMA work and would otherwise wait on memory latency every K tile
         self.stages = STAGES_SHORT if tm < 4 else 2
@@ -128,14 +151,18 @@ class Variant:
         self.b_stage = TR_STAGE if b_tr else KC_STAGE
         self.b_base = self.stages * self.a_stage   # LDS offset of B buffer 0
         self.swap = not out_f32                  # bf16: lanes own 4 consecutive columns
-        self.name = "%s%s_%s_m%d" % ("t" if a_tr else "k", "t" if b_tr else "k", "f32" if out_f32 else "bf16", 64 * tm)
+        self.name = "%s%s_%s_m%d%s" % ("t" if a_tr else "k", "t" if b_tr else "k", "f32" if out_f32 else "bf16", 64 * tm,
+                                       "_w8" if waves == 8 else "")
+
+    def acc(self, i, j):
+        return (self.tn * i + j) * 16
 
     # -- fragment reads of k16 step `s` of buffer `buf` into register set `st`; returns list of instr
     def frag_reads(self, buf, s, st):
         out = []
         for op, tr, vbase, vaddr, vbuf, stage, nblk in (
             ("A", self.a_tr, V_AF[st], V_RA, V_BUFA, self.a_stage, self.tm),
-            ("B", self.b_tr, V_BF[st], V_RB, V_BUFB, self.b_stage, 4),
+            ("B", self.b_tr, V_BF[st], V_RB, V_BUFB, self.b_stage, self.tn),
         ):
             # two buffers: the buffer is an immediate offset; three: one address register per buffer and
             # step (set up by the prologue), because the offsets no longer fit the 16-bit immediate
@@ -161,10 +188,10 @@ class Variant:
     def mfmas(self, st):
         out = []
         for i in range(self.tm):
-            for j in range(4):
+            for j in range(self.tn):
                 a = vr(V_AF[st] + 4 * i, 4)
                 b = vr(V_BF[st] + 4 * j, 4)
-                c = "a[%d:%d]" % (acc(i, j), acc(i, j) + 15)
+                c = "a[%d:%d]" % (self.acc(i, j), self.acc(i, j) + 15)
                 x, y = (b, a) if self.swap else (a, b)
                 out.append("v_mfma_f32_32x32x16_bf16 %s, %s, %s, %s" % (c, x, y, c))
         return out
@@ -190,6 +217,8 @@ class Variant:
             src = vr(vo)
         elif DBG_NO_COPY:
             return []
+        elif DBG_COPY_OOB:
+            src = vr(V_OOB)
         elif DBG_NO_MASK:
             src = vr((V_VOA if is_a else V_VOB) + i)
         else:
@@ -246,6 +275,7 @@ def interleave(e, mfmas, side_groups):
 
 
 def gen_variant(v):
+    use_regmap(v.waves)
     e = Emit()
     L = "%s_%%=" % v.name  # unique label suffix per asm instance
     sT = S_T
@@ -283,7 +313,7 @@ def gen_variant(v):
     # wave part of the LDS copy destinations: wave id is in s[S_SPARE]
     e("s_mul_i32 %s, %s, %d" % (sr(s_waveA), sr(sT + 19), v.na * (TR_BLOCK if v.a_tr else 1024)))
     e("s_add_u32 %s, %s, %s" % (sr(s_waveA), sr(s_waveA), sr(S_LDS)))
-    e("s_mul_i32 %s, %s, %d" % (sr(s_waveB), sr(sT + 19), 8 * (TR_BLOCK if v.b_tr else 1024)))
+    e("s_mul_i32 %s, %s, %d" % (sr(s_waveB), sr(sT + 19), v.nb * (TR_BLOCK if v.b_tr else 1024)))
     e("s_add_u32 %s, %s, %s" % (sr(s_waveB), sr(s_waveB), sr(S_LDS)))
     # tile 0 -> buffer 0 (head offsets)
     for n in range(v.ncopy):
@@ -312,7 +342,7 @@ def gen_variant(v):
             for ins in v.dma(n, tix, "loop", s_tail, s_oob, s_ka, s_kb, V_TMP + (n % 8)):
                 e(ins)
     # zero the accumulators while the copies fly
-    for r in range(64 * v.tm):
+    for r in range(16 * v.tm * v.tn):
         e("v_accvgpr_write_b32 a%d, 0" % r)
     e("s_waitcnt vmcnt(%d)" % ((S - 2) * v.ncopy + c3))
     e("s_barrier")
@@ -359,6 +389,8 @@ def gen_variant(v):
         cb = (buf + S - 1) % S   # buffer of tile kt + S - 1
         # step 0: MFMA set 0, read step 1 -> set 1, next copies of tile kt + S - 1
         e("s_waitcnt lgkmcnt(0)")
+        if DBG_NO_READS:
+            v.frag_reads = lambda *a: []
         side = [[x] for x in v.frag_reads(buf, 1, 1)]
         side += [v.dma(n, cb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)]
         interleave(e, v.mfmas(0), side)
@@ -381,7 +413,7 @@ def gen_variant(v):
             npf = 2
         interleave(e, v.mfmas(0), side)
         # tile kt+1 has landed for this wave; after the barrier for all, and `buf` is free
-        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % ((S - 2) * v.ncopy + npf))
+        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % (DBG_VMCNT if DBG_VMCNT >= 0 else (S - 2) * v.ncopy + npf))
         if not DBG_NO_BARRIER:
             e("s_barrier")
         if not (v.a_tr and v.b_tr):
@@ -420,49 +452,59 @@ def gen_variant(v):
     e("s_barrier")
     if not v.out_f32:
         # acc block (i, j), register 4 q + r  ->  C[m = 32 i + lane % 32][n = 32 j + 8 q + 4 (lane / 32) + r]
+        # The wave stages its block in LDS (rows padded to `pitch` bytes), `ipp` MFMA block rows per pass, and
+        # reads it back so that each lane holds 16 consecutive bytes of a row.
+        # v[V_EPI + 2] = store offset of the lane's row in read-back instruction 0 (or OOB when the lane's
+        #                columns are invalid); v[V_EPI + 3] = that row - row_lo, valid iff (unsigned) < S_ROWCNT
         t = V_TMP
-        k = 0
-        for i in range(v.tm):
-            for j in range(4):
-                for q in range(4):
-                    b = t + 6 * (k % 4)
-                    k += 1
-                    a0 = acc(i, j) + 4 * q
-                    for r in range(4):
-                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), a0 + r))
-                    e("v_cvt_pk_bf16_f32 %s, %s, %s" % (vr(b + 4), vr(b), vr(b + 1)))
-                    e("v_cvt_pk_bf16_f32 %s, %s, %s" % (vr(b + 5), vr(b + 2), vr(b + 3)))
-                    e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 4, 2), (32 * i) * PITCH + (32 * j + 8 * q) * 2))
-        e("s_waitcnt lgkmcnt(0)")
-        # read back: instruction r covers rows 4 r .. 4 r + 3 (16 lanes of 16 bytes per row)
-        # v[V_EPI + 2] = store offset of row 0 (or OOB when the lane's columns are invalid)
-        # v[V_EPI + 3] = (row of this lane at r = 0) - row_lo ; valid iff (unsigned)(that + 4 r) < S_ROWCNT
+        pitch = PITCH if v.waves == 4 else PITCH8
+        ipp = v.tm if v.waves == 4 else 2
+        rpi = 16 // v.tn          # rows per read-back instruction (64 lanes x 16 bytes over rows of 32 tn columns)
         depth = 4
-        regs = [t + 4 * x for x in range(depth)]          # data, 4 regs each (64..79)
-        voff, vrow, vsel = t + 16, t + 17, t + 18
+        regs = [t + 4 * x for x in range(depth)]          # read-back data, 4 registers each
+        voff, vrow, vsel = t + 24, t + 25, t + 26
         e("v_mov_b32 %s, %s" % (vr(voff), vr(V_EPI + 2)))
         e("v_mov_b32 %s, %s" % (vr(vrow), vr(V_EPI + 3)))
-        nrb = 8 * v.tm   # read-back instructions: 4 rows each
-        for r in range(depth):
-            e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r], 4), vr(V_EPI + 1), r * 4 * PITCH))
-        for r in range(nrb):
-            e("s_waitcnt lgkmcnt(%d)" % min(depth - 1, nrb - 1 - r))
-            e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
-            e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vsel), vr(V_OOB), vr(voff)))
-            e("buffer_store_dwordx4 %s, %s, %s, 0 offen" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
-            if r + depth < nrb:
-                # the store above must have read its data before the register is reloaded
-                e("s_nop 0")
-                e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r % depth], 4), vr(V_EPI + 1), (r + depth) * 4 * PITCH))
-            e("v_add_u32 %s, %s, %s" % (vr(voff), sr(S_CSTEP), vr(voff)))
-            e("v_add_u32 %s, 4, %s" % (vr(vrow), vr(vrow)))
+        for p0 in range(0, v.tm, ipp):
+            k = 0
+            for il in range(min(ipp, v.tm - p0)):
+                i = p0 + il
+                for j in range(v.tn):
+                    for q in range(4):
+                        b = t + 6 * (k % 4)
+                        k += 1
+                        a0 = v.acc(i, j) + 4 * q
+                        for r in range(4):
+                            e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), a0 + r))
+                        e("v_cvt_pk_bf16_f32 %s, %s, %s" % (vr(b + 4), vr(b), vr(b + 1)))
+                        e("v_cvt_pk_bf16_f32 %s, %s, %s" % (vr(b + 5), vr(b + 2), vr(b + 3)))
+                        e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 4, 2), (32 * il) * pitch + (32 * j + 8 * q) * 2))
+            e("s_waitcnt lgkmcnt(0)")
+            nrb = min(ipp, v.tm - p0) * 32 // rpi   # read-back instructions of this pass
+            for r in range(min(depth, nrb)):
+                e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r], 4), vr(V_EPI + 1), r * rpi * pitch))
+            for r in range(nrb):
+                e("s_waitcnt lgkmcnt(%d)" % min(depth - 1, nrb - 1 - r))
+                e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
+                e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vsel), vr(V_OOB), vr(voff)))
+                e("buffer_store_dwordx4 %s, %s, %s, 0 offen" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
+                if r + depth < nrb:
+                    # the store above must have read its data before the register is reloaded
+                    e("s_nop 0")
+                    e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r % depth], 4), vr(V_EPI + 1), (r + depth) * rpi * pitch))
+                e("v_add_u32 %s, %s, %s" % (vr(voff), sr(S_CSTEP), vr(voff)))
+                e("v_add_u32 %s, %d, %s" % (vr(vrow), rpi, vr(vrow)))
+            if p0 + ipp < v.tm:
+                # the next pass overwrites the staging area and the read-back registers: reads are done
+                # (lgkmcnt 0 above); the last stores must have fetched their data
+                e("s_nop 4")
     else:
         # acc block (i, j), register 4 q + r -> C[m = 32 i + 8 q + 4 (lane / 32) + r][n = 32 j + lane % 32]
         # v[V_EPI + 2] = store offset of (row 4 (lane / 32), col lane % 32); v[V_EPI + 3] = 4 (lane / 32) - row_lo
         # column validity of block j: lane mask pairs s[S_T + 24 + 2 j]
         t = V_TMP
         voff, vrow, vsel = t + 16, t + 17, t + 18
-        for j in range(4):
+        for j in range(v.tn):
             e("v_add_u32 %s, %d, %s" % (vr(t + 19), 32 * j, vr(V_EPI + 1)))   # V_EPI + 1 = lane % 32 (column in block)
             e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_NVALID), vr(t + 19)))
             e("s_mov_b64 %s, vcc" % sr(S_T + 24 + 2 * j, 2))
@@ -476,10 +518,10 @@ def gen_variant(v):
                     e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
                     e("s_mov_b64 %s, vcc" % sr(S_T + 32, 2))
                     e("s_mul_i32 %s, %s, %d" % (sr(S_T + 16), sr(S_CSTEP), row))
-                    for j in range(4):
+                    for j in range(v.tn):
                         b = t + (k % 8)
                         k += 1
-                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b), acc(i, j) + 4 * q + r))
+                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b), v.acc(i, j) + 4 * q + r))
                         e("s_and_b64 vcc, %s, %s" % (sr(S_T + 32, 2), sr(S_T + 24 + 2 * j, 2)))
                         e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(t + 8 + (k % 8)), vr(V_OOB), vr(V_EPI + 2)))
                         e("buffer_store_dword %s, %s, %s, %s offen offset:%d" % (vr(b), vr(t + 8 + (k % 8)), sr(S_RC, 4), sr(S_T + 16), 128 * j))
@@ -489,10 +531,10 @@ def gen_variant(v):
     return e
 
 
-def clobbers():
+def clobbers(v):
     c = ["memory", "vcc", "scc"]
-    c += ["v%d" % i for i in range(0, 122)] + ["v%d" % V_OOB]
-    c += ["a%d" % i for i in range(256)]
+    c += ["v%d" % i for i in range(0, V_CLOBBER)] + ["v%d" % V_OOB]
+    c += ["a%d" % i for i in range(16 * 4 * v.tn)]
     c += ["s%d" % i for i in range(S_T, S_T + 34)]
     return ", ".join('"%s"' % x for x in c)
 
@@ -507,23 +549,30 @@ def main():
     out.append("#define GMM_TILE_TR_STAGE %d" % TR_STAGE)
     out.append("#define GMM_TILE_STAGING_BYTES %d" % STAGE_BYTES)
     out.append("#define GMM_TILE_STAGES_SHORT %d" % STAGES_SHORT)
-    for a_tr, b_tr, f32, tm in [(a, b, f, t) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1)]:
-        if a_tr and tm != 4:
+    out.append("#define GMM_TILE_PITCH8 %d" % PITCH8)
+    for a_tr, b_tr, f32, tm, waves in [(a, b, f, t, w) for w in (4, 8) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1)]:
+        if tm != 4 and (a_tr or waves == 8):
             continue
-        if True:
-            if True:
-                v = Variant(a_tr, b_tr, f32, tm)
-                e = gen_variant(v)
-                out.append("")
-                out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm))
-                out.append("  asm volatile(")
-                out.append(e.text())
-                out.append('      : "={s[92:99]}"(r.stamps)' if DBG_TIMING else "      :")
-                out.append('      : "{v[128:135]}"(r.voa_head), "{v[136:143]}"(r.vob_head), "{v[144:151]}"(r.voa), "{v[152:159]}"(r.vob),')
-                out.append('        "{v[160:167]}"(r.voa_tail), "{v[168:175]}"(r.vob_tail), "{v[176:179]}"(r.ra_addr), "{v[180:183]}"(r.rb_addr),')
-                out.append('        "{v[184:187]}"(r.epi), "{v[192:193]}"(r.pf), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
-                out.append("      : %s);" % clobbers())
-                out.append("}")
+        v = Variant(a_tr, b_tr, f32, tm, waves)
+        e = gen_variant(v)
+        out.append("")
+        if waves == 4:
+            out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm))
+        else:
+            out.append("template <> __device__ __forceinline__ void gmm_tile_asm8<%d, %d, %d>(GmmTileRegs8& r) {" % (a_tr, b_tr, f32))
+        out.append("  asm volatile(")
+        out.append(e.text())
+        out.append('      : "={s[92:99]}"(r.stamps)' if DBG_TIMING else "      :")
+        if waves == 4:
+            out.append('      : "{v[128:135]}"(r.voa_head), "{v[136:143]}"(r.vob_head), "{v[144:151]}"(r.voa), "{v[152:159]}"(r.vob),')
+            out.append('        "{v[160:167]}"(r.voa_tail), "{v[168:175]}"(r.vob_tail), "{v[176:179]}"(r.ra_addr), "{v[180:183]}"(r.rb_addr),')
+            out.append('        "{v[184:187]}"(r.epi), "{v[192:193]}"(r.pf), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
+        else:
+            out.append('      : "{v[80:83]}"(r.voa_head), "{v[84:87]}"(r.vob_head), "{v[88:91]}"(r.voa), "{v[92:95]}"(r.vob),')
+            out.append('        "{v[96:99]}"(r.voa_tail), "{v[100:103]}"(r.vob_tail), "{v[104:107]}"(r.ra_addr), "{v[108:111]}"(r.rb_addr),')
+            out.append('        "{v[112:115]}"(r.epi), "{v[116:119]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
+        out.append("      : %s);" % clobbers(v))
+        out.append("}")
     sys.stdout.write("\n".join(out) + "\n")
 
 

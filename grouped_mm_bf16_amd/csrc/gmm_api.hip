@@ -267,9 +267,9 @@ int64_t gmm_host_tile_list2(const int32_t* offs_host, int32_t G, int32_t jagged,
   const int tn = gmm_cdiv(N, tile_n);
   std::vector<int32_t> ct(size_t(G) + 1, 0), cs(size_t(G) + 1, 0);
   for (int g = 0; g < G; ++g) {
-    int lo = 0, hi = 0, n_tall, n_short;
+    int lo = 0, hi = 0, n_tall, n_short, rem_rows;
     if (jagged != GMM_JAG_NONE) gmm_group_range(offs_host, g, extent, lo, hi);
-    gmm_split_rows(gmm_group_rows(jagged, lo, hi, M, align), tall, shrt, n_tall, n_short);
+    gmm_split_rows(gmm_group_rows(jagged, lo, hi, M, align), tall, shrt, n_tall, n_short, rem_rows);
     ct[g + 1] = ct[g] + n_tall * tn;
     cs[g + 1] = cs[g] + n_short * tn;
   }

@@ -119,8 +119,8 @@ __device__ __forceinline__ int gmm_build_tile_table2(const GmmParams& p, int bn,
   const int tid = threadIdx.x;
   const int tn = gmm_cdiv(p.N, bn);
   if (p.jag == GMM_JAG_NONE) {
-    int n_tall, n_short;
-    gmm_split_rows(p.M, p.tall, p.shrt, n_tall, n_short);
+    int n_tall, n_short, rem_rows;
+    gmm_split_rows(p.M, p.tall, p.shrt, n_tall, n_short, rem_rows);
     total_tall = p.G * n_tall * tn;
     return total_tall + p.G * n_short * tn;
   }
@@ -128,9 +128,9 @@ __device__ __forceinline__ int gmm_build_tile_table2(const GmmParams& p, int bn,
   for (int g = tid; g < GMM_MAX_GROUPS; g += NT) {
     int ct = 0, cs = 0;
     if (g < p.G) {
-      int lo, hi, n_tall, n_short;
+      int lo, hi, n_tall, n_short, rem_rows;
       gmm_group_range(p.offs, g, extent, lo, hi);
-      gmm_split_rows(gmm_group_rows(p.jag, lo, hi, p.M, p.align), p.tall, p.shrt, n_tall, n_short);
+      gmm_split_rows(gmm_group_rows(p.jag, lo, hi, p.M, p.align), p.tall, p.shrt, n_tall, n_short, rem_rows);
       ct = n_tall * tn;
       cs = n_short * tn;
     }
@@ -153,8 +153,8 @@ __device__ __forceinline__ GmmTile gmm_locate_tile2(const GmmParams& p, const in
   const int tc = cls ? t - total_tall : t;
   int g, local, lo = 0, hi = 0;
   if (p.jag == GMM_JAG_NONE) {
-    int n_tall, n_short;
-    gmm_split_rows(p.M, p.tall, p.shrt, n_tall, n_short);
+    int n_tall, n_short, rem_rows;
+    gmm_split_rows(p.M, p.tall, p.shrt, n_tall, n_short, rem_rows);
     const int per = (cls ? n_short : n_tall) * gmm_cdiv(p.N, bn);
     g = tc / per;
     local = tc - g * per;

@@ -263,12 +263,15 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) gmm_mfma_kernel(cons
 // contiguous along M / N (not along K) and is read from LDS with transposing loads.
 // TALL_TM: height of the tall tiles in units of 64 rows (4 or 2); 64-row short tiles for group remainders
 // exist when A is contiguous along K (p.shrt == 64).
-template <int A_TR, int B_TR, int OUT_F32, int TALL_TM>
+template <int A_TR, int B_TR, int OUT_F32>
 __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
-  constexpr int LDS_TALL = gmm_tile_lds_bytes<A_TR, B_TR, TALL_TM>();
-  constexpr int LDS_SHORT = A_TR ? 0 : gmm_tile_lds_bytes<0, B_TR, 1>();
+  // tiles of 256, 128 and 64 rows share the launch (a column-major A has only the first)
+  constexpr int LDS_256 = gmm_tile_lds_bytes<A_TR, B_TR, 4>();
+  constexpr int LDS_128 = A_TR ? 0 : gmm_tile_lds_bytes<0, B_TR, 2>();
+  constexpr int LDS_64 = A_TR ? 0 : gmm_tile_lds_bytes<0, B_TR, 1>();
+  constexpr int LDS_MAX = LDS_256 > LDS_128 ? (LDS_256 > LDS_64 ? LDS_256 : LDS_64) : (LDS_128 > LDS_64 ? LDS_128 : LDS_64);
   constexpr int BATCH = 32;  // tiles located at a time
-  __shared__ __attribute__((aligned(1024))) char lds[LDS_TALL > LDS_SHORT ? LDS_TALL : LDS_SHORT];
+  __shared__ __attribute__((aligned(1024))) char lds[LDS_MAX];
   __shared__ int32_t cum_tall[GMM_MAX_GROUPS + 1];
   __shared__ int32_t cum_short[GMM_MAX_GROUPS + 1];
   __shared__ int32_t tiles[BATCH][10];
@@ -345,7 +348,8 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       if constexpr (A_TR) {
         gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane, wave);
       } else {
-        if (rows == 64 * TALL_TM) gmm_tile_compute<A_TR, B_TR, OUT_F32, TALL_TM>(dsc, lds_base, lane, wave);
+        if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane, wave);
+        else if (rows == 128) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2>(dsc, lds_base, lane, wave);
         else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1>(dsc, lds_base, lane, wave);
       }
     }
@@ -354,17 +358,17 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
   }
 }
 
-template <int OUT_F32, int TALL_TM>
+template <int OUT_F32>
 int launch_asm(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
   const dim3 grid(p.num_wg), block(256);
   if (lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32, TALL_TM>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32>), grid, block, 0, stream, p);
   else if (lay.a_kc && !lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32, TALL_TM>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32>), grid, block, 0, stream, p);
   else if (!lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32, 4>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32, 4>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 1;
 }
 
@@ -397,8 +401,8 @@ int gmm_launch_mfma(GmmParams p, GmmLayout lay, int out_dtype, int config, int n
     // a column-major A has only the 256-row tile
     if (!lay.a_kc) { p.tall = 256; p.shrt = 0; }
     if (p.tall != 128) p.tall = 256;
-    if (out_dtype == GMM_DT_BF16) return p.tall == 256 ? launch_asm<0, 4>(p, lay, stream) : launch_asm<0, 2>(p, lay, stream);
-    if (out_dtype == GMM_DT_F32) return p.tall == 256 ? launch_asm<1, 4>(p, lay, stream) : launch_asm<1, 2>(p, lay, stream);
+    if (out_dtype == GMM_DT_BF16) return launch_asm<0>(p, lay, stream);
+    if (out_dtype == GMM_DT_F32) return launch_asm<1>(p, lay, stream);
     return -1;
   }
   if (out_dtype == GMM_DT_BF16) return launch_layout<256, 256, 2, 2, uint16_t>(p, lay, stream);

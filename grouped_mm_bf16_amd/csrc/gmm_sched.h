@@ -43,8 +43,8 @@ struct GmmParams {
   int64_t c_sg, c_sm, c_sn;
   int32_t xcd_remap;  // 1: renumber tiles so that each XCD works on a compact block
   int32_t num_wg;     // persistent grid size
-  int32_t tall;       // two-height tile list: rows of a "tall" tile (256 or 128) ...
-  int32_t shrt;       // ... and of a "short" tile for group remainders (64), or 0: tall tiles only
+  int32_t tall;       // tile list with several heights: rows of a "tall" tile (256 or 128) ...
+  int32_t shrt;       // ... and of the shortest tile for group remainders (64), or 0: tall tiles only
 };
 
 GMM_HD int gmm_cdiv(int a, int b) { return (a + b - 1) / b; }
@@ -114,19 +114,25 @@ GMM_HD int gmm_find_group(const int32_t* cum, int G, int t) {
   return lo;
 }
 
-// ---- two tile heights ------------------------------------------------------------------------ //
+// ---- tile heights ------------------------------------------------------------------------------ //
 // Skewed group sizes leave many groups far smaller than a tall tile.  The row range of a group is cut
-// into tall tiles; a remainder that fits one 64-row "short" tile becomes one (it streams B at the same
-// rate but wastes no MFMA work on rows that do not exist), a longer one pays for another tall tile: a
-// short tile runs at about half the speed per row, so two of them cost as much as a tall one.  All tall
-// tiles of all groups come first in the tile order, the short ones fill the tail of the launch.
-GMM_HD void gmm_split_rows(int rows, int tall, int shrt, int& n_tall, int& n_short) {
+// into tall tiles; a remainder that fits one shorter tile (64 rows, or 128 under 256-row tall tiles)
+// becomes one: it streams B at the same rate but wastes less MFMA work on rows that do not exist.  A
+// shorter tile runs slower per row (a 128-row tile costs about 0.6, a 64-row tile about 0.35 of a 256-row
+// one), so a remainder that needs two of them pays for another tall tile instead.  All tall tiles of
+// all groups come first in the tile order, the remainder tiles fill the tail of the launch.
+// `rem_rows` is the height of the group's remainder tile (n_short is 0 or 1).
+GMM_HD void gmm_split_rows(int rows, int tall, int shrt, int& n_tall, int& n_short, int& rem_rows) {
+  rem_rows = shrt;
   if (rows <= 0) { n_tall = 0; n_short = 0; return; }
   if (shrt <= 0) { n_tall = gmm_cdiv(rows, tall); n_short = 0; return; }
   n_tall = rows / tall;
+  n_short = 0;
   const int rem = rows - n_tall * tall;
-  if (rem > shrt) { n_tall += 1; n_short = 0; }
-  else n_short = rem > 0 ? 1 : 0;
+  if (rem == 0) return;
+  if (rem <= shrt) { n_short = 1; }
+  else if (tall > 2 * shrt && rem <= 2 * shrt) { n_short = 1; rem_rows = 2 * shrt; }
+  else n_tall += 1;
 }
 
 // Rows of group g that the tile grid has to span (from the aligned-down start when rows are jagged).
@@ -158,24 +164,20 @@ GMM_HD GmmTile gmm_make_tile(const GmmParams& p, int g, int lo, int hi, int mt, 
   return t;
 }
 
-// Tile of the two-height list: `cls` 0 = tall, 1 = short; `local` = index inside the group's tiles of
+// Tile of the list above: `cls` 0 = tall, 1 = remainder tile; `local` = index inside the group's tiles of
 // that class.  Not used with jagged columns.
 GMM_HD GmmTile gmm_make_tile2(const GmmParams& p, int g, int lo, int hi, int cls, int local, int bn) {
   const int rows = gmm_group_rows(p.jag, lo, hi, p.M, p.align);
-  int n_tall, n_short;
-  gmm_split_rows(rows, p.tall, p.shrt, n_tall, n_short);
+  int n_tall, n_short, rem_rows;
+  gmm_split_rows(rows, p.tall, p.shrt, n_tall, n_short, rem_rows);
   const int tn = gmm_cdiv(p.N, bn);
-  int mt, nt, m_off;
+  int mt = 0, nt = local, m_off = n_tall * p.tall;
   if (cls == 0) {
     gmm_decode_in_group(local, n_tall, tn, mt, nt);
     m_off = mt * p.tall;
-  } else {
-    mt = local % n_short;
-    nt = local / n_short;
-    m_off = n_tall * p.tall + mt * p.shrt;
   }
   GmmTile t = gmm_make_tile(p, g, lo, hi, 0, nt, p.tall, bn);
   t.m0 += m_off;
-  t.rows = cls == 0 ? p.tall : p.shrt;
+  t.rows = cls == 0 ? p.tall : rem_rows;
   return t;
 }

@@ -165,7 +165,7 @@ def test_two_heights_jagged_rows_exact_cover(sizes, tall, shrt, align):
     rec = tile_list2(sizes, ROWS, M, N, 16, tall, shrt, align, remap=1, num_wg=16)
     assert (coverage2(rec, len(sizes), M, N, False) == 1).all()
     heights = set(int(r[9]) for r in rec)
-    assert heights <= {tall, shrt}
+    assert heights <= {tall, 2 * shrt, shrt}
     # tall tiles come first in the launch order when ids are not renumbered
     plain = tile_list2(sizes, ROWS, M, N, 16, tall, shrt, align)
     hs = [int(r[9]) for r in plain]
@@ -176,7 +176,9 @@ def test_two_heights_jagged_rows_exact_cover(sizes, tall, shrt, align):
             rem = sz % tall
             mine = [r for r in plain if r[0] == g and r[2] == 0]
             if 0 < rem <= shrt:
-                assert sum(1 for r in mine if r[9] == shrt) == 1
+                assert sorted(int(r[9]) for r in mine) == [shrt] + [tall] * (sz // tall)
+            elif tall == 4 * shrt and 0 < rem <= 2 * shrt:
+                assert sorted(int(r[9]) for r in mine) == [2 * shrt] + [tall] * (sz // tall)
             else:
                 assert all(r[9] == tall for r in mine)
 
