@@ -107,7 +107,7 @@ int run(Problem& pr, hipStream_t stream) {
     p.xcd_remap = g_xcd_remap.load(std::memory_order_relaxed);
     const bool can_asm = asm_tile_eligible(pr, lay);
     int cfg = g_forced_config.load(std::memory_order_relaxed);
-    if (cfg == GMM_CFG_ASM_256x256 && !can_asm) return GMM_ERR_UNSUPPORTED;
+    if ((cfg == GMM_CFG_ASM_256x256 || cfg == GMM_CFG_ASM8_256x256) && !can_asm) return GMM_ERR_UNSUPPORTED;
     if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = can_asm ? GMM_CFG_ASM_256x256 : GMM_CFG_REG_256x256;
     // Tile heights of the assembly tile: 256-row tiles unless the launch would not even fill four rounds
     // of the grid, then 128; 64-row tiles for group remainders whenever A is contiguous along K.

@@ -263,12 +263,14 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) gmm_mfma_kernel(cons
 // contiguous along M / N (not along K) and is read from LDS with transposing loads.
 // TALL_TM: height of the tall tiles in units of 64 rows (4 or 2); 64-row short tiles for group remainders
 // exist when A is contiguous along K (p.shrt == 64).
-template <int A_TR, int B_TR, int OUT_F32>
-__global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
-  // tiles of 256, 128 and 64 rows share the launch (a column-major A has only the first)
+// WAVES = 4: one wave per SIMD, tiles of 256, 128 and 64 rows share the launch (a column-major A has only
+// the first).  WAVES = 8: two waves per SIMD, 256-row tiles only (the launcher sets p.shrt = 0).
+template <int A_TR, int B_TR, int OUT_F32, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams p) {
+  constexpr bool SHORT_TILES = !A_TR && WAVES == 4;
   constexpr int LDS_256 = gmm_tile_lds_bytes<A_TR, B_TR, 4>();
-  constexpr int LDS_128 = A_TR ? 0 : gmm_tile_lds_bytes<0, B_TR, 2>();
-  constexpr int LDS_64 = A_TR ? 0 : gmm_tile_lds_bytes<0, B_TR, 1>();
+  constexpr int LDS_128 = SHORT_TILES ? gmm_tile_lds_bytes<0, B_TR, 2>() : 0;
+  constexpr int LDS_64 = SHORT_TILES ? gmm_tile_lds_bytes<0, B_TR, 1>() : 0;
   constexpr int LDS_MAX = LDS_256 > LDS_128 ? (LDS_256 > LDS_64 ? LDS_256 : LDS_64) : (LDS_128 > LDS_64 ? LDS_128 : LDS_64);
   constexpr int BATCH = 32;  // tiles located at a time
   __shared__ __attribute__((aligned(1024))) char lds[LDS_MAX];
@@ -281,7 +283,7 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
   constexpr int ESZ = OUT_F32 ? 4 : 2;
 
   int total_tall;
-  const int total = gmm_build_tile_table2<256>(p, GMM_TILE_N, cum_tall, cum_short, total_tall);
+  const int total = gmm_build_tile_table2<WAVES * 64>(p, GMM_TILE_N, cum_tall, cum_short, total_tall);
   const uint16_t* __restrict__ A = static_cast<const uint16_t*>(p.a);
   const uint16_t* __restrict__ B = static_cast<const uint16_t*>(p.b);
   char* __restrict__ C = static_cast<char*>(p.c);
@@ -345,7 +347,9 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       dsc.row_cnt = gmm_min(m_hi, m0 + rows) - m_lo;
       dsc.col_lo = gmm_max(n_lo - n0, 0);
       dsc.col_hi = gmm_min(n_hi - n0, GMM_TILE_N);
-      if constexpr (A_TR) {
+      if constexpr (WAVES == 8) {
+        gmm_tile_compute8<A_TR, B_TR, OUT_F32>(dsc, lds_base, lane, wave);
+      } else if constexpr (A_TR) {
         gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane, wave);
       } else {
         if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane, wave);
@@ -358,17 +362,17 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
   }
 }
 
-template <int OUT_F32>
+template <int OUT_F32, int WAVES>
 int launch_asm(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
-  const dim3 grid(p.num_wg), block(256);
+  const dim3 grid(p.num_wg), block(WAVES * 64);
   if (lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32, WAVES>), grid, block, 0, stream, p);
   else if (lay.a_kc && !lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32, WAVES>), grid, block, 0, stream, p);
   else if (!lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32, WAVES>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32, WAVES>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 1;
 }
 
@@ -401,8 +405,15 @@ int gmm_launch_mfma(GmmParams p, GmmLayout lay, int out_dtype, int config, int n
     // a column-major A has only the 256-row tile
     if (!lay.a_kc) { p.tall = 256; p.shrt = 0; }
     if (p.tall != 128) p.tall = 256;
-    if (out_dtype == GMM_DT_BF16) return launch_asm<0>(p, lay, stream);
-    if (out_dtype == GMM_DT_F32) return launch_asm<1>(p, lay, stream);
+    if (out_dtype == GMM_DT_BF16) return launch_asm<0, 4>(p, lay, stream);
+    if (out_dtype == GMM_DT_F32) return launch_asm<1, 4>(p, lay, stream);
+    return -1;
+  }
+  if (config == GMM_CFG_ASM8_256x256) {
+    p.tall = 256;
+    p.shrt = 0;
+    if (out_dtype == GMM_DT_BF16) return launch_asm<0, 8>(p, lay, stream);
+    if (out_dtype == GMM_DT_F32) return launch_asm<1, 8>(p, lay, stream);
     return -1;
   }
   if (out_dtype == GMM_DT_BF16) return launch_layout<256, 256, 2, 2, uint16_t>(p, lay, stream);

@@ -94,7 +94,8 @@ int gmm_3d2d(const void* a, const void* b, void* out, const int32_t* offs, int32
  * (GMM_PATH_GENERIC or GMM_PATH_MFMA, 0 before any launch). */
 int gmm_set_path(int path);
 int gmm_last_path(void);
-/* Tile configuration of the MFMA family: -1 = choose from the shapes. */
+/* Tile configuration of the MFMA family: -1 = choose from the shapes, 0 = register-staged kernel,
+ * 1 = assembly tile with 4 waves (256 / 128 / 64-row tiles), 2 = assembly tile with 8 waves (256-row tiles). */
 int gmm_set_mfma_config(int config);
 int gmm_last_mfma_config(void);
 /* 0 / 1: renumber tiles per XCD (default 1). */

@@ -183,6 +183,65 @@ def test_all_layouts_all_variants_mfma(variant, a_col, b_col):
     check(out, a, b, offs, k, path="mfma")
 
 
+@pytest.mark.parametrize("a_col", [False, True])
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("variant", ["2d3d", "3d3d", "2d2d"])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_eight_wave_tile_all_layouts(variant, a_col, b_col, out_dtype):
+    """Tile configuration 2: the 256 x 256 tile computed by 8 waves (two per SIMD)."""
+    gen = torch.Generator().manual_seed(23)
+    sizes = [77, 0, 1, 330, 64, 200]  # sum 672
+    offs = offs_of(sizes)
+    G = len(sizes)
+    if variant == "2d3d":
+        a, b, shape, k, fn = rnd(gen, 672, 200), rnd(gen, G, 200, 520), (672, 520), 200, K_.grouped_mm_2d3d
+    elif variant == "3d3d":
+        a, b, shape, k, fn, offs = rnd(gen, 3, 304, 200), rnd(gen, 3, 200, 264), (3, 304, 264), 200, K_.grouped_mm_3d3d, None
+    else:
+        a, b, shape, k, fn = rnd(gen, 264, 672), rnd(gen, 672, 272), (G, 264, 272), 330, K_.grouped_mm_2d2d
+    ad, bd = a.to(DEV), b.to(DEV)
+    if a_col:
+        ad = ad.transpose(-2, -1).contiguous().transpose(-2, -1)
+    if b_col:
+        bd = bd.transpose(-2, -1).contiguous().transpose(-2, -1)
+    out = torch.full(shape, float("nan"), device=DEV, dtype=out_dtype)
+    with K_.forced_mfma_config(2):
+        if offs is None:
+            fn(ad, bd, out)
+        else:
+            fn(ad, bd, offs.to(DEV), out)
+        torch.cuda.synchronize()
+        assert K_._lib.load().gmm_last_mfma_config() == 2
+    want = oracle.grouped_mm(a, b, offs, out_dtype=out_dtype)
+    got = out.cpu()
+    assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs"
+    oracle.assert_close(got, want, k)
+
+
+@pytest.mark.parametrize("tall,shrt", [(256, 64), (256, 0), (128, 64), (128, 0)])
+@pytest.mark.parametrize("b_col", [False, True])
+def test_tile_heights_agree_bit_for_bit(tall, shrt, b_col):
+    """Groups whose remainders fall in every height class (1..64, 65..128, 129..255 rows): each forced
+    choice of tile heights gives the oracle's result, and all choices give the same bits (the order of
+    the K loop does not depend on the tile height)."""
+    gen = torch.Generator().manual_seed(29)
+    sizes = [256 + 1, 64, 65, 128, 129, 512 + 200, 0, 255, 3 * 256, 63]
+    m = sum(sizes)
+    a, b = rnd(gen, m, 328), rnd(gen, len(sizes), 328, 264, scale=0.05)
+    ad, bd, offs = a.to(DEV), b.to(DEV), offs_of(sizes)
+    if b_col:
+        bd = bd.transpose(1, 2).contiguous().transpose(1, 2)
+    outs = []
+    for heights in ((tall, shrt), (256, 0)):
+        out = torch.full((m, 264), float("nan"), device=DEV, dtype=torch.bfloat16)
+        with K_.forced_tile_heights(*heights):
+            K_.grouped_mm_2d3d(ad, bd, offs.to(DEV), out)
+        torch.cuda.synchronize()
+        outs.append(out.cpu())
+    check(outs[0], a, b, offs, 328, path="mfma")
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+
+
 def test_row_major_and_column_major_b_agree_bit_for_bit():
     gen = torch.Generator().manual_seed(19)
     a, b = rnd(gen, 4, 256, 512).to(DEV), rnd(gen, 4, 512, 256, scale=0.02).to(DEV)
