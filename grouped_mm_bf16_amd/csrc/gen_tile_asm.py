@@ -79,6 +79,7 @@ REGMAPS = {
             V_RA=176, V_RB=180,  # fragment read addresses (4 + 4)
             V_EPI=184,           # +0: stage write addr, +1: stage read addr, +2: store voffset, +3: row - row_lo
             V_OOB=188,           # constant 0x80000000
+            V_EPI2=190,          # +0: store voffset whatever the chunk's validity, +1: mask of valid elements if partial
             V_PF=192,            # A / B prefetch offsets
             V_PFD=96,            # dummy destinations of the prefetch loads (96, 97)
             V_BUFA=98, V_BUFB=110,  # three-buffer variants: fragment addresses per (buffer, step), 12 + 12
@@ -89,7 +90,7 @@ REGMAPS = {
             V_TMP=48,            # 48..79
             V_VOA_HEAD=80, V_VOB_HEAD=84, V_VOA=88, V_VOB=92, V_VOA_TAIL=96, V_VOB_TAIL=100,
             V_RA=104, V_RB=108, V_EPI=112, V_FIX=116, V_OOB=120,
-            V_PF=None, V_PFD=None, V_BUFA=None, V_BUFB=None,
+            V_PF=None, V_PFD=None, V_BUFA=None, V_BUFB=None, V_EPI2=None,
             V_CLOBBER=80),
 }
 
@@ -350,7 +351,8 @@ def gen_variant(v):
     has_kc = not (v.a_tr and v.b_tr)
     if has_kc:
         # partial first / last chunk of a jagged k range (tile 0 is also the last tile when nk == 1)
-        e("s_cmp_eq_u32 %s, 0" % sr(s_flags))
+        e("s_and_b32 %s, %s, 3" % (sr(s_t1), sr(s_flags)))
+        e("s_cmp_eq_u32 %s, 0" % sr(s_t1))
         e("s_cbranch_scc1 L_nofix0_%s" % L)
         e("s_bitcmp1_b32 %s, 0" % sr(s_flags))
         e("s_cbranch_scc0 L_nohead_%s" % L)
@@ -465,6 +467,22 @@ def gen_variant(v):
         voff, vrow, vsel = t + 24, t + 25, t + 26
         e("v_mov_b32 %s, %s" % (vr(voff), vr(V_EPI + 2)))
         e("v_mov_b32 %s, %s" % (vr(vrow), vr(V_EPI + 3)))
+        partial = v.waves == 4
+        if partial:
+            # A group boundary that is not a multiple of 8 columns leaves 16-byte chunks of which only some
+            # elements belong to this tile (flag bit 2 of the tile): those go out as 2-byte stores.
+            # eoff[e] = 2 e if element e of the lane's chunk is valid, else the out-of-range offset
+            eoff, vpoff, vtmp = t + 27, t + 35, t + 36
+            e("s_bitcmp1_b32 %s, 2" % sr(S_T + 18))
+            e("s_cbranch_scc0 L_nopart_setup_%s" % L)
+            e("v_mov_b32 %s, %s" % (vr(vpoff), vr(V_EPI2)))
+            for el in range(8):
+                e("v_bfe_u32 %s, %s, %d, 1" % (vr(vtmp), vr(V_EPI2 + 1), el))
+                e("v_cmp_ne_u32 vcc, 0, %s" % vr(vtmp))
+                e("v_mov_b32 %s, %d" % (vr(vtmp), 2 * el))
+                e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(eoff + el), vr(V_OOB), vr(vtmp)))
+            e.label("L_nopart_setup_%s" % L)
+        nstore = 0
         for p0 in range(0, v.tm, ipp):
             k = 0
             for il in range(min(ipp, v.tm - p0)):
@@ -488,6 +506,17 @@ def gen_variant(v):
                 e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
                 e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vsel), vr(V_OOB), vr(voff)))
                 e("buffer_store_dwordx4 %s, %s, %s, 0 offen" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
+                if partial:
+                    e("s_bitcmp1_b32 %s, 2" % sr(S_T + 18))
+                    e("s_cbranch_scc0 L_nopart%d_%s" % (nstore, L))
+                    for el in range(8):
+                        e("v_add_u32 %s, %s, %s" % (vr(vtmp), vr(eoff + el), vr(vpoff)))
+                        e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vtmp + 1 + el % 2), vr(V_OOB), vr(vtmp)))
+                        e("buffer_store_short%s %s, %s, %s, 0 offen" % ("_d16_hi" if el % 2 else "", vr(regs[r % depth] + el // 2),
+                                                                         vr(vtmp + 1 + el % 2), sr(S_RC, 4)))
+                    e("v_add_u32 %s, %s, %s" % (vr(vpoff), sr(S_CSTEP), vr(vpoff)))
+                    e.label("L_nopart%d_%s" % (nstore, L))
+                    nstore += 1
                 if r + depth < nrb:
                     # the store above must have read its data before the register is reloaded
                     e("s_nop 0")
@@ -566,7 +595,7 @@ def main():
         if waves == 4:
             out.append('      : "{v[128:135]}"(r.voa_head), "{v[136:143]}"(r.vob_head), "{v[144:151]}"(r.voa), "{v[152:159]}"(r.vob),')
             out.append('        "{v[160:167]}"(r.voa_tail), "{v[168:175]}"(r.vob_tail), "{v[176:179]}"(r.ra_addr), "{v[180:183]}"(r.rb_addr),')
-            out.append('        "{v[184:187]}"(r.epi), "{v[192:193]}"(r.pf), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
+            out.append('        "{v[184:187]}"(r.epi), "{v[190:191]}"(r.epi2), "{v[192:193]}"(r.pf), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
         else:
             out.append('      : "{v[80:83]}"(r.voa_head), "{v[84:87]}"(r.vob_head), "{v[88:91]}"(r.voa), "{v[92:95]}"(r.vob),')
             out.append('        "{v[96:99]}"(r.voa_tail), "{v[100:103]}"(r.vob_tail), "{v[104:107]}"(r.ra_addr), "{v[108:111]}"(r.rb_addr),')

@@ -67,7 +67,6 @@ bool mfma_eligible(const Problem& pr, GmmLayout& lay, int& align) {
 // The generated-assembly tile takes a subset of what the register-staged kernel takes.
 bool asm_tile_eligible(const Problem& pr, const GmmLayout& lay) {
   const GmmParams& p = pr.p;
-  if (p.jag == GMM_JAG_N) return false;                           // jagged columns: element-masked stores
   if (p.c_sn != 1) return false;
   const int64_t lda = lay.a_kc ? p.a_sm : p.a_sk, ldb = lay.b_kc ? p.b_sn : p.b_sk, ldc = p.c_sm;
   const int64_t ld_max = int64_t(1) << 22;
@@ -109,12 +108,17 @@ int run(Problem& pr, hipStream_t stream) {
     int cfg = g_forced_config.load(std::memory_order_relaxed);
     if ((cfg == GMM_CFG_ASM_256x256 || cfg == GMM_CFG_ASM8_256x256) && !can_asm) return GMM_ERR_UNSUPPORTED;
     if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = can_asm ? GMM_CFG_ASM_256x256 : GMM_CFG_REG_256x256;
+    // the 8-wave tile has no element-masked stores for group boundaries inside a 16-byte chunk
+    if (cfg == GMM_CFG_ASM8_256x256 && p.jag == GMM_JAG_N) return GMM_ERR_UNSUPPORTED;
+    // the assembly tile stores 16-byte chunks: its tile columns start at multiples of 8 elements
+    if (cfg == GMM_CFG_ASM_256x256 && p.jag == GMM_JAG_N) p.align = 8;
     // Tile heights of the assembly tile: 256-row tiles unless the launch would not even fill four rounds
     // of the grid, then 128; 64-row tiles for group remainders whenever A is contiguous along K.
     {
       const int64_t tn = (p.N + 255) / 256;
-      int64_t est = (p.jag == GMM_JAG_M) ? (int64_t(p.M) / 256 + (p.G < p.M ? p.G : p.M)) * tn
-                                         : int64_t(p.G) * ((p.M + 255) / 256) * tn;
+      int64_t est = int64_t(p.G) * ((p.M + 255) / 256) * tn;
+      if (p.jag == GMM_JAG_M) est = (int64_t(p.M) / 256 + (p.G < p.M ? p.G : p.M)) * tn;
+      if (p.jag == GMM_JAG_N) est = (int64_t(p.N) / 256 + (p.G < p.N ? p.G : p.N)) * ((p.M + 255) / 256);
       p.tall = (lay.a_kc && est < 4 * int64_t(cus)) ? 128 : 256;
       p.shrt = lay.a_kc ? 64 : 0;
       const int ft = g_forced_tall.load(std::memory_order_relaxed), fs = g_forced_short.load(std::memory_order_relaxed);
@@ -256,20 +260,20 @@ int64_t gmm_host_tile_list(const int32_t* offs_host, int32_t G, int32_t jagged, 
 int64_t gmm_host_tile_list2(const int32_t* offs_host, int32_t G, int32_t jagged, int32_t M, int32_t N, int32_t K,
                             int32_t tall, int32_t shrt, int32_t tile_n, int32_t align, int32_t xcd_remap,
                             int32_t num_workgroups, int32_t* records, int64_t capacity) {
-  if (G < 0 || jagged < 0 || jagged > 3 || jagged == GMM_JAG_N || tall <= 0 || shrt < 0 || tile_n <= 0 || align <= 0)
+  if (G < 0 || jagged < 0 || jagged > 3 || tall <= 0 || shrt < 0 || tile_n <= 0 || align <= 0)
     return -GMM_ERR_BAD_ARGUMENT;
   if (jagged != GMM_JAG_NONE && (!offs_host || G < 1 || G >= GMM_MAX_GROUPS)) return -GMM_ERR_BAD_ARGUMENT;
   if (xcd_remap && (num_workgroups <= 0 || num_workgroups % 8)) return -GMM_ERR_BAD_ARGUMENT;
   GmmParams p{};
   p.offs = offs_host;
   p.G = G; p.jag = jagged; p.M = M; p.N = N; p.K = K; p.align = align; p.tall = tall; p.shrt = shrt;
-  const int extent = jagged == GMM_JAG_M ? M : K;
-  const int tn = gmm_cdiv(N, tile_n);
+  const int extent = jagged == GMM_JAG_M ? M : (jagged == GMM_JAG_N ? N : K);
   std::vector<int32_t> ct(size_t(G) + 1, 0), cs(size_t(G) + 1, 0);
   for (int g = 0; g < G; ++g) {
     int lo = 0, hi = 0, n_tall, n_short, rem_rows;
     if (jagged != GMM_JAG_NONE) gmm_group_range(offs_host, g, extent, lo, hi);
     gmm_split_rows(gmm_group_rows(jagged, lo, hi, M, align), tall, shrt, n_tall, n_short, rem_rows);
+    const int tn = gmm_group_tile_cols(jagged, lo, hi, N, align, tile_n);
     ct[g + 1] = ct[g] + n_tall * tn;
     cs[g + 1] = cs[g] + n_short * tn;
   }

@@ -117,20 +117,21 @@ template <int NT>
 __device__ __forceinline__ int gmm_build_tile_table2(const GmmParams& p, int bn, int32_t* cum_tall, int32_t* cum_short,
                                                      int& total_tall) {
   const int tid = threadIdx.x;
-  const int tn = gmm_cdiv(p.N, bn);
   if (p.jag == GMM_JAG_NONE) {
+    const int tn = gmm_cdiv(p.N, bn);
     int n_tall, n_short, rem_rows;
     gmm_split_rows(p.M, p.tall, p.shrt, n_tall, n_short, rem_rows);
     total_tall = p.G * n_tall * tn;
     return total_tall + p.G * n_short * tn;
   }
-  const int extent = p.jag == GMM_JAG_M ? p.M : p.K;
+  const int extent = p.jag == GMM_JAG_M ? p.M : (p.jag == GMM_JAG_N ? p.N : p.K);
   for (int g = tid; g < GMM_MAX_GROUPS; g += NT) {
     int ct = 0, cs = 0;
     if (g < p.G) {
       int lo, hi, n_tall, n_short, rem_rows;
       gmm_group_range(p.offs, g, extent, lo, hi);
       gmm_split_rows(gmm_group_rows(p.jag, lo, hi, p.M, p.align), p.tall, p.shrt, n_tall, n_short, rem_rows);
+      const int tn = gmm_group_tile_cols(p.jag, lo, hi, p.N, p.align, bn);
       ct = n_tall * tn;
       cs = n_short * tn;
     }
@@ -162,7 +163,7 @@ __device__ __forceinline__ GmmTile gmm_locate_tile2(const GmmParams& p, const in
     const int32_t* cum = cls ? cum_short : cum_tall;
     g = gmm_find_group(cum, p.G, tc);
     local = tc - cum[g];
-    gmm_group_range(p.offs, g, p.jag == GMM_JAG_M ? p.M : p.K, lo, hi);
+    gmm_group_range(p.offs, g, p.jag == GMM_JAG_M ? p.M : (p.jag == GMM_JAG_N ? p.N : p.K), lo, hi);
   }
   return gmm_make_tile2(p, g, lo, hi, cls, local, bn);
 }

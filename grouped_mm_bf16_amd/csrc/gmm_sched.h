@@ -141,6 +141,12 @@ GMM_HD int gmm_group_rows(int jag, int lo, int hi, int M, int align) {
   return hi > lo ? hi - (lo / align) * align : 0;
 }
 
+// Tile columns of group g (from the aligned-down start when columns are jagged).
+GMM_HD int gmm_group_tile_cols(int jag, int lo, int hi, int N, int align, int bn) {
+  if (jag != GMM_JAG_N) return gmm_cdiv(N, bn);
+  return hi > lo ? gmm_cdiv(hi - (lo / align) * align, bn) : 0;
+}
+
 // One output tile, in global coordinates of the operands.
 struct GmmTile {
   int32_t g;
@@ -165,12 +171,12 @@ GMM_HD GmmTile gmm_make_tile(const GmmParams& p, int g, int lo, int hi, int mt, 
 }
 
 // Tile of the list above: `cls` 0 = tall, 1 = remainder tile; `local` = index inside the group's tiles of
-// that class.  Not used with jagged columns.
+// that class.
 GMM_HD GmmTile gmm_make_tile2(const GmmParams& p, int g, int lo, int hi, int cls, int local, int bn) {
   const int rows = gmm_group_rows(p.jag, lo, hi, p.M, p.align);
   int n_tall, n_short, rem_rows;
   gmm_split_rows(rows, p.tall, p.shrt, n_tall, n_short, rem_rows);
-  const int tn = gmm_cdiv(p.N, bn);
+  const int tn = gmm_group_tile_cols(p.jag, lo, hi, p.N, p.align, bn);
   int mt = 0, nt = local, m_off = n_tall * p.tall;
   if (cls == 0) {
     gmm_decode_in_group(local, n_tall, tn, mt, nt);

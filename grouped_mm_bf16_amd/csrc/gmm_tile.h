@@ -15,6 +15,8 @@ struct GmmTileRegs {
   gmm_v8i voa_tail, vob_tail;  // copy offsets of the last K tile
   gmm_v4i ra_addr, rb_addr;    // LDS fragment read addresses
   gmm_v4i epi;                 // epilogue: per-lane addresses (see gen_tile_asm.py)
+  gmm_v2i epi2;                // bf16 epilogue: store offset of the lane's chunk whatever its validity; mask of
+                               // its valid elements when only some of them are (a group boundary inside it)
   gmm_v2i pf;                  // L2 prefetch offsets of this lane for A and B
   gmm_v4i fix;                 // LDS addresses of this thread's row in the first / last k chunk (A, A, B, B)
   gmm_v8i masks;               // keep-masks of the first and of the last 16-byte k chunk
@@ -157,22 +159,34 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   // L2 prefetch: 256 cache lines per operand and K tile, one per lane
   r.pf[0] = A_TR ? (wave * 16 + (lane >> 2)) * t.a.ld * 2 + (lane & 3) * 128 : (wave * 64 + lane) * t.a.ld * 2;
   r.pf[1] = B_TR ? (wave * 16 + (lane >> 2)) * t.b.ld * 2 + (lane & 3) * 128 : (wave * 64 + lane) * t.b.ld * 2;
-  int c_step, n_valid = 0;
+  int c_step, n_valid = 0, partial = 0;
+  r.epi2[0] = 0;
+  r.epi2[1] = 0;
   if (!OUT_F32) {
     const int row_t = wm * WROWS + (lane >> 4), col_t = wn * 128 + (lane & 15) * 8;
     r.epi[0] = lds_base + wave * (WROWS * GMM_TILE_PITCH) + (lane & 31) * GMM_TILE_PITCH + 8 * (lane >> 5);
     r.epi[1] = lds_base + wave * (WROWS * GMM_TILE_PITCH) + (lane >> 4) * GMM_TILE_PITCH + (lane & 15) * 16;
-    r.epi[2] = (col_t >= t.col_lo && col_t + 8 <= t.col_hi) ? (row_t * t.ldc + col_t) * 2 : (int)GMM_OOB;
+    // the lane's 8 columns: all valid -> one 16-byte store; some valid (a group boundary that is not a
+    // multiple of 8 columns) -> element stores under the mask; none -> nothing
+    int mask = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mask |= (col_t + e >= t.col_lo && col_t + e < t.col_hi) ? (1 << e) : 0;
+    const int off = (row_t * t.ldc + col_t) * 2;
+    r.epi[2] = mask == 0xff ? off : (int)GMM_OOB;
     r.epi[3] = t.row_rel0 + row_t;
+    r.epi2[0] = off;
+    r.epi2[1] = mask == 0xff ? 0 : mask;
+    partial = ((t.col_lo | t.col_hi) & 7) ? 1 : 0;
     c_step = 4 * t.ldc * 2;
   } else {
+    // column c of the wave's block is valid iff (unsigned)(c - col_lo) < col_hi - col_lo
     const int row_t = wm * WROWS + 4 * (lane >> 5), col_t = wn * 128 + (lane & 31);
     r.epi[0] = 0;
-    r.epi[1] = lane & 31;
+    r.epi[1] = col_t - t.col_lo;
     r.epi[2] = (row_t * t.ldc + col_t) * 4;
     r.epi[3] = t.row_rel0 + row_t;
     c_step = t.ldc * 4;
-    n_valid = t.col_hi - wn * 128;
+    n_valid = t.col_hi - t.col_lo;
     if (n_valid < 0) n_valid = 0;
   }
   r.rsrc_a = gmm_make_rsrc(t.a.base, t.a.bytes);
@@ -184,6 +198,7 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   const int ktail = t.klen & 7;
   int flags = 0;
   if (!(A_TR && B_TR)) flags = (t.khead ? 1 : 0) | (ktail ? 2 : 0);
+  flags |= partial << 2;
   {
     // one row of each operand tile per thread (A tiles shorter than 256 rows: several threads per row,
     // all writing the same masked value)

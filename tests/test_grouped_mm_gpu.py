@@ -242,6 +242,34 @@ def test_tile_heights_agree_bit_for_bit(tall, shrt, b_col):
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
 
 
+@pytest.mark.parametrize("a_col", [False, True])
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("sizes", [[77, 0, 1, 330, 64, 200], [8, 16, 256, 512, 24], [3, 5, 7, 9, 300, 1, 600]])
+def test_3d2d_on_the_assembly_tile(sizes, out_dtype, a_col, b_col):
+    """Jagged columns: group boundaries inside a 16-byte chunk of the output go out as element stores;
+    nothing outside a group's columns (and nothing past the last offset) is written."""
+    gen = torch.Generator().manual_seed(31 + len(sizes))
+    G, n_total = len(sizes), sum(sizes)
+    extra = 16 + (-n_total % 8)   # columns past the last offset belong to nobody; the total is a multiple of 8
+    a, b = rnd(gen, G, 328, 200), rnd(gen, 200, n_total + extra, scale=0.05)
+    offs = offs_of(sizes)
+    ad, bd = a.to(DEV), b.to(DEV)
+    if a_col:
+        ad = ad.transpose(-2, -1).contiguous().transpose(-2, -1)
+    if b_col:
+        bd = bd.transpose(-2, -1).contiguous().transpose(-2, -1)
+    out = torch.full((328, n_total + extra), float("nan"), device=DEV, dtype=out_dtype)
+    K_.grouped_mm_3d2d(ad, bd, offs.to(DEV), out)
+    torch.cuda.synchronize()
+    assert K_.last_path() == "mfma" and K_._lib.load().gmm_last_mfma_config() == 1
+    got = out.cpu()
+    assert torch.isnan(got[:, n_total:].float()).all()
+    want = oracle.grouped_mm(a, b, offs, out_dtype=out_dtype)
+    assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs"
+    oracle.assert_close(got, want, 200)
+
+
 def test_row_major_and_column_major_b_agree_bit_for_bit():
     gen = torch.Generator().manual_seed(19)
     a, b = rnd(gen, 4, 256, 512).to(DEV), rnd(gen, 4, 512, 256, scale=0.02).to(DEV)

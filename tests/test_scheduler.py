@@ -183,6 +183,21 @@ def test_two_heights_jagged_rows_exact_cover(sizes, tall, shrt, align):
                 assert all(r[9] == tall for r in mine)
 
 
+@pytest.mark.parametrize("sizes", SIZE_LISTS + [[129, 128, 127, 65, 64, 63, 1, 700]])
+@pytest.mark.parametrize("tall,shrt,align", [(256, 64, 8), (128, 64, 8), (256, 0, 8), (256, 64, 1)])
+def test_two_heights_jagged_columns_exact_cover(sizes, tall, shrt, align):
+    """3D x 2D on the assembly tile: rows are split by height, every group has its own tile columns, and
+    tile columns start at multiples of `align` elements."""
+    N, M = sum(sizes), 330
+    if N == 0:
+        return
+    rec = tile_list2(sizes, COLS, M, N, 16, tall, shrt, align, remap=1, num_wg=16)
+    assert (coverage2(rec, len(sizes), M, N, False) == 1).all()
+    for g, m0, n0, m_lo, m_hi, n_lo, n_hi, _, _, rows in rec:
+        assert n0 % align == 0 and n0 <= max(n_lo, n0) and (m_lo, m_hi) == (0, M)
+        assert rows in (tall, 2 * shrt, shrt)
+
+
 @pytest.mark.parametrize("tall,shrt", [(256, 64), (128, 64), (256, 0)])
 def test_two_heights_contraction_and_batched(tall, shrt):
     sizes = [7, 0, 1, 13, 11]
