@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the copy-kernel
 # calibration); see profiles/.  None where no profile has been taken.
 MEASURED_TRAFFIC = {"mixtral": 4102504356, "fine": 594652279, "batched": 671390287, "batched_colmajor": None,
-                    "kgrouped": 7042960350}
+                    "kgrouped": 7042960350, "ngrouped": None}
 
 
 def load_sizes(key):
@@ -77,6 +77,14 @@ def make_workload(name, torch):
                  flops=2.0 * 4096 * 16384 * 14336, bound="mfma", k=16384,
                  bytes=a.numel() * 2 + b.numel() * 2 + 8 * 4096 * 14336 * 4,
                  desc="k_grouped_weight_grad_2d2d_G8_M4096_Ktotal16384_N14336_fp32out")
+    elif name == "ngrouped":
+        sizes = load_sizes("mixtral_top2_g8")
+        a = torch.randn(8, 4096, 4096, generator=g1).to(bf)
+        b = (torch.randn(4096, 16384, generator=g2) * 0.02).to(bf)
+        w = dict(variant="3d2d", sizes=sizes, a=a, b=b, out_shape=(4096, 16384), out_dtype=bf,
+                 flops=2.0 * 4096 * 4096 * 16384, bound="mfma", k=4096,
+                 bytes=a.numel() * 2 + b.numel() * 2 + 4096 * 16384 * 2,
+                 desc="n_grouped_3d2d_G8_M4096_K4096_Ntotal16384_skewed_top2")
     else:
         raise SystemExit(f"unknown workload {name}")
     w["launch"] = {"2d3d": kernels.grouped_mm_2d3d, "3d3d": kernels.grouped_mm_3d3d,
@@ -129,6 +137,8 @@ def cpu_baseline(w, torch, budget_s=15.0):
         # batched / K-grouped: a slab of the first group
         if w["variant"] == "3d3d":
             x, y = a[0].float(), b[0].float()
+        elif w["variant"] == "3d2d":
+            x, y = a[0].float(), b[:, :sizes[0]].float()
         else:
             e = sizes[0]
             x, y = a[:, :e].float(), b[:e].float()
@@ -148,7 +158,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="mixtral",
-                    choices=["mixtral", "fine", "batched", "batched_colmajor", "kgrouped", "copy"])
+                    choices=["mixtral", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--path", default="auto", choices=["auto", "mfma", "generic"])
     args = ap.parse_args()
