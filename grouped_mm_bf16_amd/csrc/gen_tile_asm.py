@@ -58,6 +58,7 @@ DBG_NO_BARRIER = int(os.environ.get("GMM_GEN_DBG_NO_BARRIER", "0"))
 DBG_COPY_OOB = int(os.environ.get("GMM_GEN_DBG_COPY_OOB", "0"))  # timing only: loop copies fetch nothing (write zeros)
 DBG_NO_READS = int(os.environ.get("GMM_GEN_DBG_NO_READS", "0"))  # timing only: no fragment reads in the loop
 DBG_NO_MASK = int(os.environ.get("GMM_GEN_DBG_NO_MASK", "0"))
+FAST_PATH = int(os.environ.get("GMM_GEN_FAST_PATH", "1"))  # interior K tiles without the per-copy tail / range selects
 DBG_VMCNT = int(os.environ.get("GMM_GEN_DBG_VMCNT", "-1"))  # timing experiments only: copies left in flight at the K-tile barrier
 DBG_TIMING = int(os.environ.get("GMM_GEN_DBG_TIMING", "0"))  # phase timestamps in s[92:99] (extra asm output)
 
@@ -213,6 +214,9 @@ class Variant:
         blk = TR_BLOCK if tr else 1024
         lds_off = lbase + buf * stage + i * blk
         s_wave = S_T + 20 + (0 if is_a else 1)
+        # m0 is written first: a write of m0 needs one other instruction before the copy that uses it
+        # (the selects below, an MFMA that interleave() puts in between, or a s_nop)
+        out.append("s_add_u32 m0, %s, %d" % (sr(s_wave), lds_off))
         if which == "head":
             vo = (V_VOA_HEAD if is_a else V_VOB_HEAD) + i
             src = vr(vo)
@@ -220,7 +224,7 @@ class Variant:
             return []
         elif DBG_COPY_OOB:
             src = vr(V_OOB)
-        elif DBG_NO_MASK:
+        elif DBG_NO_MASK or which == "fast":
             src = vr((V_VOA if is_a else V_VOB) + i)
         else:
             vn = (V_VOA if is_a else V_VOB) + i
@@ -228,10 +232,18 @@ class Variant:
             out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(vn), vr(vt), sr(s_tail, 2)))
             out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(tmp), vr(V_OOB), sr(s_oob, 2)))
             src = vr(tmp)
-        out.append("s_add_u32 m0, %s, %d" % (sr(s_wave), lds_off))
-        out.append("s_nop 0")
         out.append("buffer_load_dwordx4 %s, %s, %s offen lds" % (src, sr(S_RA if is_a else S_RB, 4), sr(s_ka if is_a else s_kb)))
         return out
+
+
+def m0_gaps(lines):
+    """Insert the wait state between a write of m0 and a copy that follows it directly."""
+    out = []
+    for ins in lines:
+        if ins.startswith("buffer_load") and out and out[-1].startswith("s_add_u32 m0"):
+            out.append("s_nop 0")
+        out.append(ins)
+    return out
 
 
 def fixup(e, v, which, buf):
@@ -262,17 +274,24 @@ def fixup(e, v, which, buf):
 
 
 def interleave(e, mfmas, side_groups):
-    """Emit 16 MFMAs with the side groups spread between them (one group after each MFMA, in order)."""
+    """Emit the MFMAs of a step with the side groups spread between them (after each MFMA, in order).  A
+    group that starts with a write of m0 has that write moved in front of the MFMA, which then is the
+    instruction the hardware wants between the write and the copy."""
     n = len(mfmas)
     slots = [[] for _ in range(n)]
     # spread groups evenly over the first n - 1 gaps
     g = len(side_groups)
     for k, grp in enumerate(side_groups):
         slots[min(n - 1, (k * n) // max(g, 1))].extend(grp)
+    lines = []
     for k in range(n):
-        e(mfmas[k])
-        for ins in slots[k]:
-            e(ins)
+        side = list(slots[k])
+        if side and side[0].startswith("s_add_u32 m0"):
+            lines.append(side.pop(0))
+        lines.append(mfmas[k])
+        lines.extend(side)
+    for ins in m0_gaps(lines):
+        e(ins)
 
 
 def gen_variant(v):
@@ -318,7 +337,7 @@ def gen_variant(v):
     e("s_add_u32 %s, %s, %s" % (sr(s_waveB), sr(s_waveB), sr(S_LDS)))
     # tile 0 -> buffer 0 (head offsets)
     for n in range(v.ncopy):
-        for ins in v.dma(n, 0, "head", 0, 0, s_zero, s_zero, V_TMP):
+        for ins in m0_gaps(v.dma(n, 0, "head", 0, 0, s_zero, s_zero, V_TMP)):
             e(ins)
     S = v.stages
     c3, c0, c1, c2 = v.sched
@@ -340,7 +359,7 @@ def gen_variant(v):
         e("s_mul_i32 %s, %s, %d" % (sr(s_ka), sr(S_ASTEP), tix))
         e("s_mul_i32 %s, %s, %d" % (sr(s_kb), sr(S_BSTEP), tix))
         for n in range(v.ncopy if tix < S - 1 else c3):
-            for ins in v.dma(n, tix, "loop", s_tail, s_oob, s_ka, s_kb, V_TMP + (n % 8)):
+            for ins in m0_gaps(v.dma(n, tix, "loop", s_tail, s_oob, s_ka, s_kb, V_TMP + (n % 8))):
                 e(ins)
     # zero the accumulators while the copies fly
     for r in range(16 * v.tm * v.tn):
@@ -375,16 +394,21 @@ def gen_variant(v):
     e("s_cbranch_scc1 L_done_%s" % L)
 
     # ------------------------------------------------------------------ K loop, two tiles per trip
-    def ktile(buf):
-        # on entry: fragments of step 0 in set 0 (in flight); copies 0..5 of tile kt+1 in flight
-        e("; ---- k tile on buffer %d" % buf)
-        # K offsets and masks of tiles kt + S - 1 (copied during steps 0..2) and kt + S (step 3)
+    def ktile(buf, fast):
+        # on entry: fragments of step 0 in set 0 (in flight); the first c3 copies of tile kt + S - 1 in flight.
+        # fast: tiles kt + S - 1 and kt + S are both before the last one, so their copies need neither the
+        # tail offsets nor the out-of-range select, and tile kt + 1 cannot be the last one.
+        which = "fast" if fast else "loop"
+        e("; ---- k tile on buffer %d%s" % (buf, " (interior)" if fast else ""))
+        # K offsets (and masks) of tiles kt + S - 1 (copied during steps 0..2) and kt + S (step 3)
         e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), S - 1))
-        tile_masks(s_t1, s_tail1, s_oob1)
+        if not fast:
+            tile_masks(s_t1, s_tail1, s_oob1)
         e("s_mul_i32 %s, %s, %s" % (sr(s_ka1), sr(s_t1), sr(S_ASTEP)))
         e("s_mul_i32 %s, %s, %s" % (sr(s_kb1), sr(s_t1), sr(S_BSTEP)))
         e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), S))
-        tile_masks(s_t1, s_tail2, s_oob2)
+        if not fast:
+            tile_masks(s_t1, s_tail2, s_oob2)
         e("s_mul_i32 %s, %s, %s" % (sr(s_ka2), sr(s_t1), sr(S_ASTEP)))
         e("s_mul_i32 %s, %s, %s" % (sr(s_kb2), sr(s_t1), sr(S_BSTEP)))
         nb = (buf + 1) % S       # buffer of tile kt + 1
@@ -394,17 +418,17 @@ def gen_variant(v):
         if DBG_NO_READS:
             v.frag_reads = lambda *a: []
         side = [[x] for x in v.frag_reads(buf, 1, 1)]
-        side += [v.dma(n, cb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)]
+        side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)]
         interleave(e, v.mfmas(0), side)
         # step 1
         e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 2, 0)]
-        side += [v.dma(n, cb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)]
+        side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)]
         interleave(e, v.mfmas(1), side)
         # step 2
         e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 3, 1)]
-        side += [v.dma(n, cb, "loop", s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)]
+        side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)]
         npf = 0
         if PREFETCH:
             e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), PREFETCH))
@@ -418,7 +442,7 @@ def gen_variant(v):
         e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % (DBG_VMCNT if DBG_VMCNT >= 0 else (S - 2) * v.ncopy + npf))
         if not DBG_NO_BARRIER:
             e("s_barrier")
-        if not (v.a_tr and v.b_tr):
+        if not (v.a_tr and v.b_tr) and not fast:
             # the tile that has just landed is the last one and its last chunk is partial
             e("s_add_u32 %s, %s, 1" % (sr(s_t1), sr(s_kt)))
             e("s_cmp_eq_u32 %s, %s" % (sr(s_t1), sr(s_last)))
@@ -431,16 +455,27 @@ def gen_variant(v):
             e.label("L_nofix%d_%s" % (buf + 1, L))
         # step 3: MFMA set 1, read step 0 of the next tile -> set 0, first copies of tile kt + S -> buf
         side = [[x] for x in v.frag_reads(nb, 0, 0)]
-        side += [v.dma(n, buf, "loop", s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, c3)]
+        side += [v.dma(n, buf, which, s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, c3)]
         interleave(e, v.mfmas(1), side)
         e("s_add_u32 %s, %s, 1" % (sr(s_kt), sr(s_kt)))
 
+    def ktile_both(buf):
+        if FAST_PATH:
+            e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), S))
+            e("s_cmp_lt_u32 %s, %s" % (sr(s_t1), sr(s_last)))
+            e("s_cbranch_scc0 L_slow%d_%s" % (buf, L))
+            ktile(buf, True)
+            e("s_branch L_join%d_%s" % (buf, L))
+            e.label("L_slow%d_%s" % (buf, L))
+        ktile(buf, False)
+        e.label("L_join%d_%s" % (buf, L))
+
     e.label("L_loop_%s" % L)
     for buf in range(S - 1):
-        ktile(buf)
+        ktile_both(buf)
         e("s_cmp_ge_u32 %s, %s" % (sr(s_kt), sr(S_NK)))
         e("s_cbranch_scc1 L_done_%s" % L)
-    ktile(S - 1)
+    ktile_both(S - 1)
     e("s_cmp_lt_u32 %s, %s" % (sr(s_kt), sr(S_NK)))
     e("s_cbranch_scc1 L_loop_%s" % L)
     e.label("L_done_%s" % L)

@@ -76,6 +76,8 @@ bool asm_tile_eligible(const Problem& pr, const GmmLayout& lay) {
   if (!lay.b_kc && int64_t(p.K) * ldb * 2 >= (int64_t(1) << 31)) return false;
   if (pr.out_dtype == GMM_DT_BF16) {
     if (!aligned16(p.c) || !mult8(p.c_sm) || !mult8(p.c_sg) || !mult8(p.N)) return false;
+  } else if (ldc >= ld_max / 2) {
+    return false;   // 255 rows of 4-byte elements must stay below 2^31 bytes from the tile's origin
   }
   return true;
 }
