@@ -317,6 +317,23 @@ def test_1023_groups_bf16_mfma():
     check(out, a, b, offs, 64, path="mfma")
 
 
+def test_1023_groups_bf16_mfma_3d2d_and_2d2d():
+    """The alternating 3 / 0 pattern of the reference's 1023-group cases on the MFMA family: every
+    group boundary of 3D x 2D lies inside a 16-byte chunk of the output."""
+    gen = torch.Generator().manual_seed(33)
+    sizes = [3 if i % 2 == 0 else 0 for i in range(1023)]
+    sizes[-1] = 0
+    tot, offs = sum(sizes), offs_of(sizes)          # 1533 columns; pad the total to a multiple of 8
+    n_total = tot + (-tot % 8)
+    a, b = rnd(gen, 1023, 16, 64), rnd(gen, 64, n_total)
+    out = run_poisoned(K_.grouped_mm_3d2d, a, b, offs, (16, n_total), torch.bfloat16)
+    check(out, a, b, offs, 64, path="mfma")
+    k_total = tot + (-tot % 8)
+    a2, b2 = rnd(gen, 16, k_total), rnd(gen, k_total, 24)
+    out2 = run_poisoned(K_.grouped_mm_2d2d, a2, b2, offs, (1023, 16, 24), torch.bfloat16)
+    check(out2, a2, b2, offs, 3, path="mfma")
+
+
 def test_fp32_epilogue_for_bf16_inputs_through_the_launcher():
     """The public function keeps the reference's dtype rule; the launcher honours out.dtype."""
     gen = torch.Generator().manual_seed(37)
