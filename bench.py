@@ -152,6 +152,29 @@ def cpu_baseline(w, torch, budget_s=15.0):
             "sample": sample, "seconds": round(t, 3)}
 
 
+def library_comparator(w, a, b, offs, torch, steps):
+    """PyTorch-ROCm's own grouped GEMM on the same device tensors: context for `value`, never an oracle."""
+    import torch.nn.functional as F
+    if not hasattr(F, "grouped_mm") or w["out_dtype"] != a.dtype:
+        return {"name": "torch.nn.functional.grouped_mm", "value": None, "note": "not applicable to this workload"}
+    run = (lambda: F.grouped_mm(a, b)) if offs is None else (lambda: F.grouped_mm(a, b, offs=offs))
+    try:
+        for _ in range(3):
+            run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+    except Exception as ex:  # the library rejects some layouts; that is a result too
+        return {"name": "torch.nn.functional.grouped_mm", "value": None, "note": repr(ex)[:200]}
+    ms = e0.elapsed_time(e1) / steps
+    return {"name": "torch.nn.functional.grouped_mm", "value": round(w["flops"] / (ms * 1e-3) / 1e12, 2),
+            "unit": "TFLOP/s", "ms_per_step": round(ms, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -160,6 +183,8 @@ def main():
     ap.add_argument("--workload", default="mixtral",
                     choices=["mixtral", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--library-comparator", action="store_true",
+                    help="also time PyTorch-ROCm's own torch.nn.functional.grouped_mm on the same tensors (context only)")
     ap.add_argument("--path", default="auto", choices=["auto", "mfma", "generic"])
     args = ap.parse_args()
     if args.gpus != 1:
@@ -256,6 +281,8 @@ def main():
                      "kernel_ms_median": round(statistics.median(k_ms), 4),
                      "algorithmic_flops": w["flops"], "algorithmic_bytes": w["bytes"]},
     }
+    if args.library_comparator:
+        rec["library_comparator"] = library_comparator(w, a, b, offs, torch, args.steps)
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(w, torch)
     print(json.dumps(rec))
