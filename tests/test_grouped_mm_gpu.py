@@ -153,6 +153,39 @@ def test_rows_past_the_last_offset_are_not_written():
         assert torch.isnan(out[23:].float()).all()
 
 
+def test_launch_replays_from_a_captured_graph():
+    """The launcher allocates nothing and never synchronises, so it can be captured; every replay must
+    give what the eager launch gives on the same inputs (new contents, same buffers)."""
+    gen = torch.Generator().manual_seed(41)
+    sizes = [130, 0, 257, 64, 61]
+    m, offs = sum(sizes), offs_of(sizes).to(DEV)
+    a_s = torch.zeros(m, 192, device=DEV, dtype=torch.bfloat16)
+    b_s = torch.zeros(len(sizes), 192, 264, device=DEV, dtype=torch.bfloat16)
+    out_s = torch.zeros(m, 264, device=DEV, dtype=torch.bfloat16)
+    K_.grouped_mm_2d3d(a_s, b_s, offs, out_s)        # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            K_.grouped_mm_2d3d(a_s, b_s, offs, out_s)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        a, b = rnd(gen, m, 192), rnd(gen, len(sizes), 192, 264)
+        a_s.copy_(a.to(DEV))
+        b_s.copy_(b.to(DEV))
+        out_s.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = out_s.clone()
+        eager = torch.full_like(out_s, float("nan"))
+        K_.grouped_mm_2d3d(a_s, b_s, offs, eager)
+        torch.cuda.synchronize()
+        assert torch.equal(replayed.view(torch.int16), eager.view(torch.int16)), f"replay {rep} differs from eager"
+        check(replayed, a, b, offs.cpu(), 192)
+
+
 # ------------------------------------------------------------------ operand layouts
 @pytest.mark.parametrize("a_col", [False, True])
 @pytest.mark.parametrize("b_col", [False, True])
