@@ -308,6 +308,11 @@ __global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams 
     const int64_t left = (int64_t(total) - blockIdx.x + gridDim.x - 1) / gridDim.x - first;  // tiles of this workgroup from `first` on
     const int here = left < BATCH ? int(left) : BATCH;
     for (int j = 0; j < here; ++j) {
+      // Everything the assembly wants per lane is a cheap function of the lane id.  Hidden from the
+      // optimiser per tile, or it hoists those values out of the loop, keeps them alive across the
+      // assembly (which clobbers most registers) and spills them to scratch memory.
+      int lane_j = lane;
+      asm volatile("" : "+v"(lane_j));
       const int32_t* d = tiles[j];
       const int g = __builtin_amdgcn_readfirstlane(d[0]);
       const int m0 = __builtin_amdgcn_readfirstlane(d[1]), n0 = __builtin_amdgcn_readfirstlane(d[2]);
@@ -348,13 +353,13 @@ __global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams 
       dsc.col_lo = gmm_max(n_lo - n0, 0);
       dsc.col_hi = gmm_min(n_hi - n0, GMM_TILE_N);
       if constexpr (WAVES == 8) {
-        gmm_tile_compute8<A_TR, B_TR, OUT_F32>(dsc, lds_base, lane, wave);
+        gmm_tile_compute8<A_TR, B_TR, OUT_F32>(dsc, lds_base, lane_j, wave);
       } else if constexpr (A_TR) {
-        gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane, wave);
+        gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane_j, wave);
       } else {
-        if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane, wave);
-        else if (rows == 128) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2>(dsc, lds_base, lane, wave);
-        else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1>(dsc, lds_base, lane, wave);
+        if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane_j, wave);
+        else if (rows == 128) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2>(dsc, lds_base, lane_j, wave);
+        else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1>(dsc, lds_base, lane_j, wave);
       }
     }
     if (left <= BATCH) break;

@@ -202,7 +202,7 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   {
     // one row of each operand tile per thread (A tiles shorter than 256 rows: several threads per row,
     // all writing the same masked value)
-    const int row = threadIdx.x, row_a = threadIdx.x % (64 * TM);
+    const int row = wave * 64 + lane, row_a = row % (64 * TM);
     const int c_last = ((t.klen - 1) & (GMM_TILE_K - 1)) >> 3;
     r.fix[0] = lds_base + row_a * 128 + ((0 ^ gmm_swz(row_a)) << 4);
     r.fix[1] = lds_base + row_a * 128 + ((c_last ^ gmm_swz(row_a)) << 4);
@@ -303,7 +303,7 @@ __device__ __forceinline__ void gmm_tile_compute8(const GmmTileDesc& t, unsigned
   if (!(A_TR && B_TR)) flags = (t.khead ? 1 : 0) | (ktail ? 2 : 0);
   {
     // one row of each operand tile per thread pair (both write the same masked value)
-    const int row = threadIdx.x & 255;
+    const int row = (wave * 64 + lane) & 255;
     const int c_last = ((t.klen - 1) & (GMM_TILE_K - 1)) >> 3;
     r.fix[0] = lds_base + row * 128 + ((0 ^ gmm_swz(row)) << 4);
     r.fix[1] = lds_base + row * 128 + ((c_last ^ gmm_swz(row)) << 4);
