@@ -58,6 +58,7 @@ DBG_NO_BARRIER = int(os.environ.get("GMM_GEN_DBG_NO_BARRIER", "0"))
 DBG_COPY_OOB = int(os.environ.get("GMM_GEN_DBG_COPY_OOB", "0"))  # timing only: loop copies fetch nothing (write zeros)
 DBG_NO_READS = int(os.environ.get("GMM_GEN_DBG_NO_READS", "0"))  # timing only: no fragment reads in the loop
 DBG_NO_MASK = int(os.environ.get("GMM_GEN_DBG_NO_MASK", "0"))
+PARTIAL_WAITS = int(os.environ.get("GMM_GEN_PARTIAL_WAITS", "1"))  # MFMAs wait for their own fragments only
 FAST_PATH = int(os.environ.get("GMM_GEN_FAST_PATH", "1"))  # interior K tiles without the per-copy tail / range selects
 DBG_VMCNT = int(os.environ.get("GMM_GEN_DBG_VMCNT", "-1"))  # timing experiments only: copies left in flight at the K-tile barrier
 DBG_TIMING = int(os.environ.get("GMM_GEN_DBG_TIMING", "0"))  # phase timestamps in s[92:99] (extra asm output)
@@ -161,7 +162,9 @@ class Variant:
 
     # -- fragment reads of k16 step `s` of buffer `buf` into register set `st`; returns list of instr
     def frag_reads(self, buf, s, st):
-        out = []
+        """Order: A block 0, all B blocks, then the other A blocks -- the order in which the MFMAs of the
+        step (block row 0 first) need them, so that they can start while later reads are still in flight."""
+        blocks = {}
         for op, tr, vbase, vaddr, vbuf, stage, nblk in (
             ("A", self.a_tr, V_AF[st], V_RA, V_BUFA, self.a_stage, self.tm),
             ("B", self.b_tr, V_BF[st], V_RB, V_BUFB, self.b_stage, self.tn),
@@ -176,12 +179,27 @@ class Variant:
                 d = vbase + 4 * x
                 if not tr:
                     # address register per step; sub-tiles are 32 rows = 4096 bytes apart
-                    out.append("ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(reg), boff + x * 4096))
+                    blocks[(op, x)] = ["ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(reg), boff + x * 4096)]
                 else:
                     o = boff + s * 8 * TR_BLOCK + x * 64
-                    out.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d, 2), vr(reg), o))
-                    out.append("ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d + 2, 2), vr(reg), o + 512))
+                    blocks[(op, x)] = ["ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d, 2), vr(reg), o),
+                                       "ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d + 2, 2), vr(reg), o + 512)]
+        self.read_order = [("A", 0)] + [("B", x) for x in range(self.tn)] + [("A", x) for x in range(1, self.tm)]
+        self.read_len = {t: len(blocks[t]) for t in self.read_order}
+        out = []
+        for t in self.read_order:
+            out += blocks[t]
         return out
+
+    def read_need(self):
+        """For every MFMA of a step (in mfmas() order): how many of the step's fragment reads, in issue
+        order, must have completed before it; and the number of reads of a step."""
+        self.frag_reads(0, 0, 0)
+        end, n = {}, 0
+        for t in self.read_order:
+            n += self.read_len[t]
+            end[t] = n
+        return [max(end[("A", i)], end[("B", j)]) for i in range(self.tm) for j in range(self.tn)], n
 
     def n_frag_reads(self):
         return 4 * (2 if self.a_tr else 1) + 4 * (2 if self.b_tr else 1)
@@ -273,10 +291,14 @@ def fixup(e, v, which, buf):
         e("ds_write_b128 %s, %s" % (vr(ta), vr(t, 4)))
 
 
-def interleave(e, mfmas, side_groups):
+def interleave(e, mfmas, side_groups, need=None, prev_total=0):
     """Emit the MFMAs of a step with the side groups spread between them (after each MFMA, in order).  A
     group that starts with a write of m0 has that write moved in front of the MFMA, which then is the
-    instruction the hardware wants between the write and the copy."""
+    instruction the hardware wants between the write and the copy.
+
+    need / prev_total: the operands of MFMA k are the first need[k] of the prev_total LDS reads issued
+    before this step (LDS reads complete in order); each MFMA waits only for those, counting the reads
+    this step has issued in the meantime (lgkmcnt has 4 bits: a larger allowance waits for 15)."""
     n = len(mfmas)
     slots = [[] for _ in range(n)]
     # spread groups evenly over the first n - 1 gaps
@@ -284,12 +306,23 @@ def interleave(e, mfmas, side_groups):
     for k, grp in enumerate(side_groups):
         slots[min(n - 1, (k * n) // max(g, 1))].extend(grp)
     lines = []
+    bound = 1 << 30   # upper bound on the LDS reads in flight, as far as the emitted waits prove it
+    issued = 0        # reads issued in this step so far
     for k in range(n):
         side = list(slots[k])
         if side and side[0].startswith("s_add_u32 m0"):
             lines.append(side.pop(0))
+        if need is not None and PARTIAL_WAITS:
+            allowed = prev_total - need[k] + issued
+            if bound > allowed:
+                w = min(allowed, 15)
+                lines.append("s_waitcnt lgkmcnt(%d)" % w)
+                bound = w
         lines.append(mfmas[k])
         lines.extend(side)
+        nr = sum(1 for x in side if x.startswith("ds_read"))
+        issued += nr
+        bound += nr
     for ins in m0_gaps(lines):
         e(ins)
 
@@ -394,6 +427,11 @@ def gen_variant(v):
     e("s_cbranch_scc1 L_done_%s" % L)
 
     # ------------------------------------------------------------------ K loop, two tiles per trip
+    need, nreads = v.read_need()
+    if DBG_NO_READS:
+        v.frag_reads = lambda *a: []
+        need, nreads = [0] * len(need), 0
+
     def ktile(buf, fast):
         # on entry: fragments of step 0 in set 0 (in flight); the first c3 copies of tile kt + S - 1 in flight.
         # fast: tiles kt + S - 1 and kt + S are both before the last one, so their copies need neither the
@@ -414,19 +452,20 @@ def gen_variant(v):
         nb = (buf + 1) % S       # buffer of tile kt + 1
         cb = (buf + S - 1) % S   # buffer of tile kt + S - 1
         # step 0: MFMA set 0, read step 1 -> set 1, next copies of tile kt + S - 1
-        e("s_waitcnt lgkmcnt(0)")
-        if DBG_NO_READS:
-            v.frag_reads = lambda *a: []
+        if not PARTIAL_WAITS:
+            e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 1, 1)]
         side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)]
-        interleave(e, v.mfmas(0), side)
+        interleave(e, v.mfmas(0), side, need, nreads)
         # step 1
-        e("s_waitcnt lgkmcnt(0)")
+        if not PARTIAL_WAITS:
+            e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 2, 0)]
         side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)]
-        interleave(e, v.mfmas(1), side)
+        interleave(e, v.mfmas(1), side, need, nreads)
         # step 2
-        e("s_waitcnt lgkmcnt(0)")
+        if not PARTIAL_WAITS:
+            e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 3, 1)]
         side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)]
         npf = 0
@@ -437,7 +476,7 @@ def gen_variant(v):
             side.append(["buffer_load_dword %s, %s, %s, %s offen" % (vr(V_PFD), vr(V_PF), sr(S_RA, 4), sr(sT + 16))])
             side.append(["buffer_load_dword %s, %s, %s, %s offen" % (vr(V_PFD + 1), vr(V_PF + 1), sr(S_RB, 4), sr(sT + 17))])
             npf = 2
-        interleave(e, v.mfmas(0), side)
+        interleave(e, v.mfmas(0), side, need, nreads)
         # tile kt+1 has landed for this wave; after the barrier for all, and `buf` is free
         e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % (DBG_VMCNT if DBG_VMCNT >= 0 else (S - 2) * v.ncopy + npf))
         if not DBG_NO_BARRIER:
