@@ -103,28 +103,42 @@ struct GmmTileDesc {
 };
 
 // NI = copy instructions per wave and K tile for this operand (8 for 256 rows, 2 per 64 rows).
+// klen, khead and nk are the same for all lanes: whether the first / last K tile is a whole one is a
+// scalar branch, and only partial ones pay for the per-lane selects.
 template <int TR, int NI>
 __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int klen, int khead, int nk,
                                                  gmm_v8i& head, gmm_v8i& full, gmm_v8i& tail) {
+  int kk[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    if (i >= NI) { head[i] = full[i] = tail[i] = (int)GMM_OOB; continue; }
-    int k, vo;
+    if (i >= NI) { kk[i] = 0; full[i] = (int)GMM_OOB; continue; }
     if (!TR) {
       const int row = wave * (NI * 8) + i * 8 + (lane >> 3);
       const int c = (lane & 7) ^ gmm_swz(row);
-      k = c * 8;
-      vo = row * ld * 2 + c * 16;
+      kk[i] = c * 8;
+      full[i] = row * ld * 2 + c * 16;
     } else {
       const int blk = wave * 8 + i;
-      k = 8 * (blk >> 2) + (blk & 3) + 4 * (lane >> 5);
-      vo = k * ld * 2 + (lane & 31) * 16;
+      kk[i] = 8 * (blk >> 2) + (blk & 3) + 4 * (lane >> 5);
+      full[i] = kk[i] * ld * 2 + (lane & 31) * 16;
     }
-    // whole k rows before the range are skipped (transposed layout); inside a chunk the fix-up masks them
-    const bool before = TR && k < khead;
-    full[i] = vo;
-    head[i] = (k < klen && !before) ? vo : (int)GMM_OOB;
-    tail[i] = ((nk - 1) * GMM_TILE_K + k < klen && !(before && nk == 1)) ? vo : (int)GMM_OOB;
+  }
+  head = full;
+  tail = full;
+  if (!(khead == 0 && klen >= GMM_TILE_K)) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      // whole k rows before the range are skipped (transposed layout); inside a chunk the fix-up masks them
+      const bool before = TR && kk[i] < khead;
+      head[i] = (kk[i] < klen && !before) ? full[i] : (int)GMM_OOB;
+    }
+  }
+  if (!(klen > 0 && (klen & (GMM_TILE_K - 1)) == 0 && !(khead != 0 && nk == 1))) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const bool before = TR && kk[i] < khead;
+      tail[i] = ((nk - 1) * GMM_TILE_K + kk[i] < klen && !(before && nk == 1)) ? full[i] : (int)GMM_OOB;
+    }
   }
 }
 
