@@ -138,8 +138,9 @@ def sr(base, n=1):
 class Variant:
     """tm = MFMA block rows per wave: the tile is 64 tm rows (256 / 128 / 64) by 256 columns."""
 
-    def __init__(self, a_tr, b_tr, out_f32, tm=4, waves=4):
-        self.a_tr, self.b_tr, self.out_f32, self.tm, self.waves = a_tr, b_tr, out_f32, tm, waves
+    def __init__(self, a_tr, b_tr, out_f32, tm=4, waves=4, f16=0):
+        self.a_tr, self.b_tr, self.out_f32, self.tm, self.waves, self.f16 = a_tr, b_tr, out_f32, tm, waves, f16
+        self.dt = "f16" if f16 else "bf16"   # element type of A, B and of a 16-bit output
         assert tm in (1, 2, 4) and (tm == 4 or not a_tr) and (waves == 4 or (waves == 8 and tm == 4 and not PREFETCH))
         self.tn = 16 // waves            # 32-column MFMA blocks per wave (the wave grid is 2 x waves / 2)
         self.na = 8 * tm // waves        # copies of the A tile per wave and K tile
@@ -154,8 +155,8 @@ class Variant:
         self.b_stage = TR_STAGE if b_tr else KC_STAGE
         self.b_base = self.stages * self.a_stage   # LDS offset of B buffer 0
         self.swap = not out_f32                  # bf16: lanes own 4 consecutive columns
-        self.name = "%s%s_%s_m%d%s" % ("t" if a_tr else "k", "t" if b_tr else "k", "f32" if out_f32 else "bf16", 64 * tm,
-                                       "_w8" if waves == 8 else "")
+        self.name = "%s%s_%s_%s_m%d%s" % ("t" if a_tr else "k", "t" if b_tr else "k", self.dt, "f32" if out_f32 else self.dt,
+                                          64 * tm, "_w8" if waves == 8 else "")
 
     def acc(self, i, j):
         return (self.tn * i + j) * 16
@@ -213,7 +214,7 @@ class Variant:
                 b = vr(V_BF[st] + 4 * j, 4)
                 c = "a[%d:%d]" % (self.acc(i, j), self.acc(i, j) + 15)
                 x, y = (b, a) if self.swap else (a, b)
-                out.append("v_mfma_f32_32x32x16_bf16 %s, %s, %s, %s" % (c, x, y, c))
+                out.append("v_mfma_f32_32x32x16_%s %s, %s, %s, %s" % (self.dt, c, x, y, c))
         return out
 
     # -- copy instruction n (0..15) of a K tile into buffer buf.
@@ -568,8 +569,8 @@ def gen_variant(v):
                         a0 = v.acc(i, j) + 4 * q
                         for r in range(4):
                             e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), a0 + r))
-                        e("v_cvt_pk_bf16_f32 %s, %s, %s" % (vr(b + 4), vr(b), vr(b + 1)))
-                        e("v_cvt_pk_bf16_f32 %s, %s, %s" % (vr(b + 5), vr(b + 2), vr(b + 3)))
+                        e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 4), vr(b), vr(b + 1)))
+                        e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 5), vr(b + 2), vr(b + 3)))
                         e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 4, 2), (32 * il) * pitch + (32 * j + 8 * q) * 2))
             e("s_waitcnt lgkmcnt(0)")
             nrb = min(ipp, v.tm - p0) * 32 // rpi   # read-back instructions of this pass
@@ -653,14 +654,15 @@ def main():
     out.append("#define GMM_TILE_STAGING_BYTES %d" % STAGE_BYTES)
     out.append("#define GMM_TILE_STAGES_SHORT %d" % STAGES_SHORT)
     out.append("#define GMM_TILE_PITCH8 %d" % PITCH8)
-    for a_tr, b_tr, f32, tm, waves in [(a, b, f, t, w) for w in (4, 8) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1)]:
-        if tm != 4 and (a_tr or waves == 8):
+    for a_tr, b_tr, f32, tm, waves, f16 in [(a, b, f, t, w, h) for h in (0, 1) for w in (4, 8) for a in (0, 1) for b in (0, 1)
+                                            for f in (0, 1) for t in (4, 2, 1)]:
+        if (tm != 4 and (a_tr or waves == 8)) or (f16 and waves == 8):
             continue
-        v = Variant(a_tr, b_tr, f32, tm, waves)
+        v = Variant(a_tr, b_tr, f32, tm, waves, f16)
         e = gen_variant(v)
         out.append("")
         if waves == 4:
-            out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm))
+            out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm, f16))
         else:
             out.append("template <> __device__ __forceinline__ void gmm_tile_asm8<%d, %d, %d>(GmmTileRegs8& r) {" % (a_tr, b_tr, f32))
         out.append("  asm volatile(")

@@ -46,8 +46,8 @@ struct Problem {
 // Decide whether the MFMA family can take the call, and with which operand layouts.
 bool mfma_eligible(const Problem& pr, GmmLayout& lay, int& align) {
   const GmmParams& p = pr.p;
-  if (pr.in_dtype != GMM_DT_BF16) return false;
-  if (pr.out_dtype != GMM_DT_BF16 && pr.out_dtype != GMM_DT_F32) return false;
+  if (pr.in_dtype != GMM_DT_BF16 && pr.in_dtype != GMM_DT_F16) return false;
+  if (pr.out_dtype != pr.in_dtype && pr.out_dtype != GMM_DT_F32) return false;
   if (!aligned16(p.a) || !aligned16(p.b)) return false;
   if (!mult8(p.a_sg) || !mult8(p.b_sg)) return false;
   // A: contiguous along K (row-major) or along M (column-major)
@@ -74,7 +74,7 @@ bool asm_tile_eligible(const Problem& pr, const GmmLayout& lay) {
   // a transposed-layout operand is addressed from its first k row: the whole slice must fit 31 bits
   if (!lay.a_kc && int64_t(p.K) * lda * 2 >= (int64_t(1) << 31)) return false;
   if (!lay.b_kc && int64_t(p.K) * ldb * 2 >= (int64_t(1) << 31)) return false;
-  if (pr.out_dtype == GMM_DT_BF16) {
+  if (pr.out_dtype != GMM_DT_F32) {
     if (!aligned16(p.c) || !mult8(p.c_sm) || !mult8(p.c_sg) || !mult8(p.N)) return false;
   } else if (ldc >= ld_max / 2) {
     return false;   // 255 rows of 4-byte elements must stay below 2^31 bytes from the tile's origin
@@ -98,7 +98,10 @@ int run(Problem& pr, hipStream_t stream) {
   GmmLayout lay{};
   int align = 1;
   const int forced = g_forced_path.load(std::memory_order_relaxed);
-  const bool can_mfma = mfma_eligible(pr, lay, align);
+  const bool aligned = mfma_eligible(pr, lay, align);
+  const bool can_asm = aligned && asm_tile_eligible(pr, lay);
+  // fp16 has the assembly tile only (configuration 1); bf16 also the register-staged kernel and the 8-wave tile
+  const bool can_mfma = aligned && (pr.in_dtype == GMM_DT_BF16 || can_asm);
   if (forced == GMM_PATH_MFMA && !can_mfma) return GMM_ERR_UNSUPPORTED;
   const bool use_mfma = can_mfma && forced != GMM_PATH_GENERIC;
 
@@ -106,10 +109,10 @@ int run(Problem& pr, hipStream_t stream) {
   if (use_mfma) {
     p.align = align;
     p.xcd_remap = g_xcd_remap.load(std::memory_order_relaxed);
-    const bool can_asm = asm_tile_eligible(pr, lay);
     int cfg = g_forced_config.load(std::memory_order_relaxed);
     if ((cfg == GMM_CFG_ASM_256x256 || cfg == GMM_CFG_ASM8_256x256) && !can_asm) return GMM_ERR_UNSUPPORTED;
     if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = can_asm ? GMM_CFG_ASM_256x256 : GMM_CFG_REG_256x256;
+    if (pr.in_dtype != GMM_DT_BF16 && cfg != GMM_CFG_ASM_256x256) return GMM_ERR_UNSUPPORTED;
     // the 8-wave tile has no element-masked stores for group boundaries inside a 16-byte chunk
     if (cfg == GMM_CFG_ASM8_256x256 && p.jag == GMM_JAG_N) return GMM_ERR_UNSUPPORTED;
     // the assembly tile stores 16-byte chunks: its tile columns start at multiples of 8 elements
@@ -127,7 +130,7 @@ int run(Problem& pr, hipStream_t stream) {
       if (lay.a_kc && (ft == 256 || ft == 128)) p.tall = ft;
       if (lay.a_kc && (fs == 0 || fs == 64)) p.shrt = fs;
     }
-    rc = gmm_launch_mfma(p, lay, pr.out_dtype, cfg, cus, stream);
+    rc = gmm_launch_mfma(p, lay, pr.in_dtype, pr.out_dtype, cfg, cus, stream);
     t_last_path = GMM_PATH_MFMA;
     t_last_config = cfg;
   } else {

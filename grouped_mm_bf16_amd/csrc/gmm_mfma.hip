@@ -265,7 +265,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) gmm_mfma_kernel(cons
 // exist when A is contiguous along K (p.shrt == 64).
 // WAVES = 4: one wave per SIMD, tiles of 256, 128 and 64 rows share the launch (a column-major A has only
 // the first).  WAVES = 8: two waves per SIMD, 256-row tiles only (the launcher sets p.shrt = 0).
-template <int A_TR, int B_TR, int OUT_F32, int WAVES>
+template <int A_TR, int B_TR, int OUT_F32, int WAVES, int F16>
 __global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams p) {
   constexpr bool SHORT_TILES = !A_TR && WAVES == 4;
   constexpr int LDS_256 = gmm_tile_lds_bytes<A_TR, B_TR, 4>();
@@ -355,11 +355,11 @@ __global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams 
       if constexpr (WAVES == 8) {
         gmm_tile_compute8<A_TR, B_TR, OUT_F32>(dsc, lds_base, lane_j, wave);
       } else if constexpr (A_TR) {
-        gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane_j, wave);
+        gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16>(dsc, lds_base, lane_j, wave);
       } else {
-        if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4>(dsc, lds_base, lane_j, wave);
-        else if (rows == 128) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2>(dsc, lds_base, lane_j, wave);
-        else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1>(dsc, lds_base, lane_j, wave);
+        if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16>(dsc, lds_base, lane_j, wave);
+        else if (rows == 128) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2, F16>(dsc, lds_base, lane_j, wave);
+        else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1, F16>(dsc, lds_base, lane_j, wave);
       }
     }
     if (left <= BATCH) break;
@@ -367,17 +367,17 @@ __global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams 
   }
 }
 
-template <int OUT_F32, int WAVES>
+template <int OUT_F32, int WAVES, int F16>
 int launch_asm(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
   const dim3 grid(p.num_wg), block(WAVES * 64);
   if (lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32, WAVES>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32, WAVES, F16>), grid, block, 0, stream, p);
   else if (lay.a_kc && !lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32, WAVES>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32, WAVES, F16>), grid, block, 0, stream, p);
   else if (!lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32, WAVES>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32, WAVES, F16>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32, WAVES>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32, WAVES, F16>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 1;
 }
 
@@ -404,24 +404,24 @@ void gmm_mfma_tile_shape(int config, int& bm, int& bn) {
   bn = 256;
 }
 
-int gmm_launch_mfma(GmmParams p, GmmLayout lay, int out_dtype, int config, int num_cus, hipStream_t stream) {
+int gmm_launch_mfma(GmmParams p, GmmLayout lay, int in_dtype, int out_dtype, int config, int num_cus, hipStream_t stream) {
   p.num_wg = num_cus;
+  const bool out16 = out_dtype == in_dtype;   // else fp32
+  if (!out16 && out_dtype != GMM_DT_F32) return -1;
   if (config == GMM_CFG_ASM_256x256) {
     // a column-major A has only the 256-row tile
     if (!lay.a_kc) { p.tall = 256; p.shrt = 0; }
     if (p.tall != 128) p.tall = 256;
-    if (out_dtype == GMM_DT_BF16) return launch_asm<0, 4>(p, lay, stream);
-    if (out_dtype == GMM_DT_F32) return launch_asm<1, 4>(p, lay, stream);
+    if (in_dtype == GMM_DT_BF16) return out16 ? launch_asm<0, 4, 0>(p, lay, stream) : launch_asm<1, 4, 0>(p, lay, stream);
+    if (in_dtype == GMM_DT_F16) return out16 ? launch_asm<0, 4, 1>(p, lay, stream) : launch_asm<1, 4, 1>(p, lay, stream);
     return -1;
   }
+  if (in_dtype != GMM_DT_BF16) return -1;     // the other configurations are bf16 only
   if (config == GMM_CFG_ASM8_256x256) {
     p.tall = 256;
     p.shrt = 0;
-    if (out_dtype == GMM_DT_BF16) return launch_asm<0, 8>(p, lay, stream);
-    if (out_dtype == GMM_DT_F32) return launch_asm<1, 8>(p, lay, stream);
-    return -1;
+    return out16 ? launch_asm<0, 8, 0>(p, lay, stream) : launch_asm<1, 8, 0>(p, lay, stream);
   }
-  if (out_dtype == GMM_DT_BF16) return launch_layout<256, 256, 2, 2, uint16_t>(p, lay, stream);
-  if (out_dtype == GMM_DT_F32) return launch_layout<256, 256, 2, 2, float>(p, lay, stream);
-  return -1;
+  if (out16) return launch_layout<256, 256, 2, 2, uint16_t>(p, lay, stream);
+  return launch_layout<256, 256, 2, 2, float>(p, lay, stream);
 }

@@ -26,7 +26,8 @@ struct GmmTileRegs {
 };
 
 // TM = MFMA block rows per wave: the tile is 64 * TM rows (256, 128 or 64) by 256 columns.
-template <int A_TR, int B_TR, int OUT_F32, int TM>
+// F16 = 1: A, B and a 16-bit output are fp16 instead of bf16 (same layouts, other MFMA and conversion).
+template <int A_TR, int B_TR, int OUT_F32, int TM, int F16>
 __device__ __forceinline__ void gmm_tile_asm(GmmTileRegs& r);
 
 // Same for the 8-wave form of the 256 x 256 tile (two waves per SIMD, 128 x 64 per wave): every wave
@@ -142,7 +143,7 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int
   }
 }
 
-template <int A_TR, int B_TR, int OUT_F32, int TM = 4>
+template <int A_TR, int B_TR, int OUT_F32, int TM = 4, int F16 = 0>
 __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave,
                                                  gmm_v8i* stamps = nullptr) {
   static_assert(TM == 4 || !A_TR, "short tiles exist for a K-contiguous A only");
@@ -233,7 +234,7 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   const int sc[8] = {nk, a_step, b_step, (int)lds_base, t.row_cnt, c_step, n_valid, wave | (flags << 8)};
 #pragma unroll
   for (int i = 0; i < 8; ++i) r.scal[i] = __builtin_amdgcn_readfirstlane(sc[i]);
-  gmm_tile_asm<A_TR, B_TR, OUT_F32, TM>(r);
+  gmm_tile_asm<A_TR, B_TR, OUT_F32, TM, F16>(r);
   if (stamps) *stamps = r.stamps;
 }
 

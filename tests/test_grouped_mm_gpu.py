@@ -322,6 +322,43 @@ def test_fp32_and_fp16_inputs(dtype, tol):
     torch.testing.assert_close(got, want, rtol=tol, atol=tol)
 
 
+@pytest.mark.parametrize("a_col", [False, True])
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("variant", ["2d3d", "3d3d", "2d2d", "3d2d"])
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
+def test_fp16_inputs_on_the_assembly_tile(variant, a_col, b_col, out_dtype):
+    """fp16 inputs take the same tile with the fp16 MFMA; fp16 or fp32 out."""
+    gen = torch.Generator().manual_seed(43)
+    sizes = [77, 0, 1, 330, 64, 200]  # sum 672
+    offs = offs_of(sizes)
+    G, h = len(sizes), torch.float16
+    if variant == "2d3d":
+        a, b, shape, k, fn = rnd(gen, 672, 200, dtype=h), rnd(gen, G, 200, 264, dtype=h), (672, 264), 200, K_.grouped_mm_2d3d
+    elif variant == "3d3d":
+        a, b, shape, k, fn, offs = rnd(gen, 3, 304, 200, dtype=h), rnd(gen, 3, 200, 264, dtype=h), (3, 304, 264), 200, K_.grouped_mm_3d3d, None
+    elif variant == "2d2d":
+        a, b, shape, k, fn = rnd(gen, 264, 672, dtype=h), rnd(gen, 672, 272, dtype=h), (G, 264, 272), 330, K_.grouped_mm_2d2d
+    else:
+        a, b, shape, k, fn = rnd(gen, G, 264, 200, dtype=h), rnd(gen, 200, 672, dtype=h), (264, 672), 200, K_.grouped_mm_3d2d
+    ad, bd = a.to(DEV), b.to(DEV)
+    if a_col:
+        ad = ad.transpose(-2, -1).contiguous().transpose(-2, -1)
+    if b_col:
+        bd = bd.transpose(-2, -1).contiguous().transpose(-2, -1)
+    out = torch.full(shape, float("nan"), device=DEV, dtype=out_dtype)
+    if offs is None:
+        fn(ad, bd, out)
+    else:
+        fn(ad, bd, offs.to(DEV), out)
+    torch.cuda.synchronize()
+    assert K_.last_path() == "mfma" and K_._lib.load().gmm_last_mfma_config() == 1
+    want = oracle.grouped_mm(a, b, offs, out_dtype=out_dtype)
+    got = out.cpu()
+    assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs"
+    # fp16 keeps 11 bits: one rounding of the fp32 sum, and the sum itself in another order than the oracle's
+    torch.testing.assert_close(got.float(), want.float(), rtol=2e-3, atol=2e-2 if out_dtype == torch.float16 else 2e-3)
+
+
 @pytest.mark.parametrize("variant", ["2d3d", "3d2d", "2d2d"])
 def test_1023_groups_fp32(variant):
     """G = 1023, sizes alternate 1, 0 with a trailing empty group (reference tests :661-747)."""
