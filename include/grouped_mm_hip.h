@@ -39,7 +39,7 @@ enum gmm_status {
 
 enum gmm_dtype { GMM_DT_BF16 = 0, GMM_DT_F16 = 1, GMM_DT_F32 = 2 };
 
-/* Kernel families.  AUTO picks MFMA when the operands qualify (bf16, 16-byte
+/* Kernel families.  AUTO picks MFMA when the operands qualify (bf16 or fp16, 16-byte
  * aligned bases and leading dimensions), else GENERIC. */
 enum gmm_path { GMM_PATH_AUTO = 0, GMM_PATH_GENERIC = 1, GMM_PATH_MFMA = 2 };
 
