@@ -383,7 +383,8 @@ def test_1023_groups_bf16_mfma():
     sizes[-1] = 0
     tot, offs = sum(sizes), offs_of(sizes)
     a, b = rnd(gen, tot, 64), rnd(gen, 1023, 64, 16)
-    out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs, (tot, 16), torch.bfloat16)
+    with K_.forced_path("mfma"):
+        out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs, (tot, 16), torch.bfloat16)
     check(out, a, b, offs, 64, path="mfma")
 
 
@@ -400,8 +401,22 @@ def test_1023_groups_bf16_mfma_3d2d_and_2d2d():
     check(out, a, b, offs, 64, path="mfma")
     k_total = tot + (-tot % 8)
     a2, b2 = rnd(gen, 16, k_total), rnd(gen, k_total, 24)
-    out2 = run_poisoned(K_.grouped_mm_2d2d, a2, b2, offs, (1023, 16, 24), torch.bfloat16)
+    with K_.forced_path("mfma"):
+        out2 = run_poisoned(K_.grouped_mm_2d2d, a2, b2, offs, (1023, 16, 24), torch.bfloat16)
     check(out2, a2, b2, offs, 3, path="mfma")
+
+
+def test_tiny_products_take_the_generic_kernel_unless_forced():
+    """K <= 128 and N <= 64 (the default shape of the reference's benchmark): a 256-column tile would
+    mostly multiply padding."""
+    gen = torch.Generator().manual_seed(47)
+    sizes = [40, 0, 24]
+    a, b, offs = rnd(gen, 64, 32), rnd(gen, 3, 32, 64), offs_of(sizes)
+    out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs, (64, 64), torch.bfloat16)
+    check(out, a, b, offs, 32, path="generic")
+    with K_.forced_path("mfma"):
+        out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs, (64, 64), torch.bfloat16)
+    check(out, a, b, offs, 32, path="mfma")
 
 
 def test_fp32_epilogue_for_bf16_inputs_through_the_launcher():
