@@ -103,10 +103,7 @@ int run(Problem& pr, hipStream_t stream) {
   // fp16 has the assembly tile only (configuration 1); bf16 also the register-staged kernel and the 8-wave tile
   const bool can_mfma = aligned && (pr.in_dtype == GMM_DT_BF16 || can_asm);
   if (forced == GMM_PATH_MFMA && !can_mfma) return GMM_ERR_UNSUPPORTED;
-  // A 256-column tile on a very narrow, very short product (the reference bench's default K = 32, N = 64)
-  // mostly multiplies padding; the 64 x 64 generic kernel is faster there.
-  const bool tiny = p.N <= 64 && p.K <= 128;
-  const bool use_mfma = can_mfma && forced != GMM_PATH_GENERIC && !(tiny && forced == GMM_PATH_AUTO);
+  const bool use_mfma = can_mfma && forced != GMM_PATH_GENERIC;
 
   int rc;
   if (use_mfma) {

@@ -99,7 +99,10 @@ int launch(const GmmParams& p, hipStream_t stream) {
 int gmm_launch_generic(GmmParams p, int in_dtype, int out_dtype, int num_cus, hipStream_t stream) {
   p.align = 1;
   p.xcd_remap = 0;
-  p.num_wg = num_cus * 4;
+  {
+    const int64_t bound = gmm_tile_bound(p.jag, p.G, p.M, p.N, 64, 64);
+    p.num_wg = int(bound < int64_t(num_cus) * 4 ? (bound < 1 ? 1 : bound) : int64_t(num_cus) * 4);
+  }
   if (in_dtype == GMM_DT_BF16 && out_dtype == GMM_DT_BF16) return launch<gmm_bf16, gmm_bf16>(p, stream);
   if (in_dtype == GMM_DT_BF16 && out_dtype == GMM_DT_F32) return launch<gmm_bf16, float>(p, stream);
   if (in_dtype == GMM_DT_F16 && out_dtype == GMM_DT_F16) return launch<gmm_f16, gmm_f16>(p, stream);

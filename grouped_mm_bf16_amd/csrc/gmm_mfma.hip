@@ -405,7 +405,13 @@ void gmm_mfma_tile_shape(int config, int& bm, int& bn) {
 }
 
 int gmm_launch_mfma(GmmParams p, GmmLayout lay, int in_dtype, int out_dtype, int config, int num_cus, hipStream_t stream) {
-  p.num_wg = num_cus;
+  // persistent grid: one workgroup per CU, fewer (a multiple of 8, for the XCD renumbering) when the launch
+  // cannot have that many tiles
+  {
+    const int64_t bound = gmm_tile_bound(p.jag, p.G, p.M, p.N, config == GMM_CFG_ASM_256x256 ? p.tall : 256, 256);
+    const int64_t want = ((bound + 7) / 8) * 8;
+    p.num_wg = int(want < num_cus ? (want < 8 ? 8 : want) : num_cus);
+  }
   const bool out16 = out_dtype == in_dtype;   // else fp32
   if (!out16 && out_dtype != GMM_DT_F32) return -1;
   if (config == GMM_CFG_ASM_256x256) {

@@ -73,6 +73,17 @@ GMM_HD void gmm_group_grid(int jag, int lo, int hi, int M, int N, int bm, int bn
   if (jag == GMM_JAG_N) tiles_n = hi > lo ? gmm_cdiv(hi - (lo / align) * align, bn) : 0;
 }
 
+// Upper bound on the number of tiles of a launch that needs no look at the offsets (the host uses it to
+// launch fewer workgroups for small problems; a grid larger than the tile count only costs start-up
+// time).  bm = smallest tile height in use.  Every group can add a partial tile at its end, one for the
+// aligned-down start and one remainder tile: three per group on top of the even split.
+GMM_HD int64_t gmm_tile_bound(int jag, int G, int M, int N, int bm, int bn) {
+  const int64_t tm = gmm_cdiv(M, bm), tn = gmm_cdiv(N, bn);
+  if (jag == GMM_JAG_M) return (int64_t(M) / bm + 3 * int64_t(G)) * tn;
+  if (jag == GMM_JAG_N) return (int64_t(N) / bn + 3 * int64_t(G)) * (tm + 1);
+  return int64_t(G) * (tm + 1) * tn;
+}
+
 // Linear id inside a group -> (tile row, tile column).  Tile rows advance
 // fastest inside bands of GMM_BAND rows, so tiles that run at the same time
 // share a few A row panels and a few B column panels.

@@ -37,13 +37,14 @@ def _require_gpu(*tensors) -> None:
             raise RuntimeError("grouped_mm_bf16 is GPU-only (CUDA/HIP); CPU tensors are not supported")
 
 
-@torch.library.custom_op("grouped_mm_bf16_amd::launch", mutates_args=("out",))
-def _launch(variant: int, a: torch.Tensor, b: torch.Tensor, offs: Optional[torch.Tensor],
-            out: torch.Tensor) -> None:
+def _launch_now(variant: int, a: torch.Tensor, b: torch.Tensor, offs: Optional[torch.Tensor],
+                out: torch.Tensor) -> None:
     lib = _lib.load()
     _require_gpu(a, b, offs, out)
     in_dt, out_dt = _dtype_code(a.dtype), _dtype_code(out.dtype)
-    with torch.cuda.device(a.device):
+    # the device guard costs microseconds; only switch when the tensors live on another device
+    guard = torch.cuda.device(a.device) if a.device.index != torch.cuda.current_device() else contextlib.nullcontext()
+    with guard:
         stream = torch.cuda.current_stream().cuda_stream
         pa, pb, po = a.data_ptr(), b.data_ptr(), out.data_ptr()
         poffs = offs.data_ptr() if offs is not None else None
@@ -66,6 +67,18 @@ def _launch(variant: int, a: torch.Tensor, b: torch.Tensor, offs: Optional[torch
         else:
             raise RuntimeError(f"unknown variant {variant}")
     _lib.check(rc, "grouped_mm launch")
+
+
+# The launch as a torch custom op (mutates `out`), for callers that trace or compile.  Eager calls skip
+# the dispatcher, which costs more than the kernel for small products.
+_launch_op = torch.library.custom_op("grouped_mm_bf16_amd::launch", mutates_args=("out",))(_launch_now)
+
+
+def _launch(variant: int, a: torch.Tensor, b: torch.Tensor, offs: Optional[torch.Tensor], out: torch.Tensor) -> None:
+    if torch.compiler.is_compiling():
+        _launch_op(variant, a, b, offs, out)
+    else:
+        _launch_now(variant, a, b, offs, out)
 
 
 def grouped_mm_3d3d(mat_a: torch.Tensor, mat_b: torch.Tensor, out: torch.Tensor) -> None:

@@ -406,19 +406,6 @@ def test_1023_groups_bf16_mfma_3d2d_and_2d2d():
     check(out2, a2, b2, offs, 3, path="mfma")
 
 
-def test_tiny_products_take_the_generic_kernel_unless_forced():
-    """K <= 128 and N <= 64 (the default shape of the reference's benchmark): a 256-column tile would
-    mostly multiply padding."""
-    gen = torch.Generator().manual_seed(47)
-    sizes = [40, 0, 24]
-    a, b, offs = rnd(gen, 64, 32), rnd(gen, 3, 32, 64), offs_of(sizes)
-    out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs, (64, 64), torch.bfloat16)
-    check(out, a, b, offs, 32, path="generic")
-    with K_.forced_path("mfma"):
-        out = run_poisoned(K_.grouped_mm_2d3d, a, b, offs, (64, 64), torch.bfloat16)
-    check(out, a, b, offs, 32, path="mfma")
-
-
 def test_fp32_epilogue_for_bf16_inputs_through_the_launcher():
     """The public function keeps the reference's dtype rule; the launcher honours out.dtype."""
     gen = torch.Generator().manual_seed(37)
