@@ -310,6 +310,62 @@ def test_row_major_and_column_major_b_agree_bit_for_bit():
     assert torch.equal(grouped_mm(a, b).view(torch.int16), grouped_mm(a, b_col).view(torch.int16))
 
 
+# ------------------------------------------------------------------ seeded random sweep
+def _random_case(rng):
+    variant = ["2d3d", "3d3d", "2d2d", "3d2d"][int(rng.integers(0, 4))]
+    G = int(rng.integers(1, 9))
+    # group sizes around the tile heights (0, 1, 63..65, 127..129, 255..257, a few hundred)
+    pool = [0, 0, 1, 2, 7, 8, 9, 31, 63, 64, 65, 100, 127, 128, 129, 191, 192, 193, 255, 256, 257, 300, 511, 513]
+    sizes = [int(pool[int(rng.integers(0, len(pool)))]) for _ in range(G)]
+    if sum(sizes) == 0:
+        sizes[0] = 8
+    mult8 = lambda x: max(8, (x + 7) // 8 * 8)
+    d1 = mult8(int(rng.integers(8, 400)))
+    d2 = mult8(int(rng.integers(8, 600)))
+    return variant, sizes, d1, d2
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_all_variants(seed):
+    """Random variant / group sizes / extents / layouts / element and output types, MFMA family, against
+    the oracle with exact ownership."""
+    rng = np.random.default_rng(1000 + seed)
+    gen = torch.Generator().manual_seed(2000 + seed)
+    for _ in range(4):
+        variant, sizes, d1, d2 = _random_case(rng)
+        G, tot = len(sizes), sum(sizes)
+        tot8 = tot + (-tot % 8)           # the jagged extent, padded so that strides stay multiples of 8
+        dt = [torch.bfloat16, torch.float16][int(rng.integers(0, 2))]
+        out_dt = [dt, torch.float32][int(rng.integers(0, 2))]
+        a_col, b_col = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        offs = offs_of(sizes)
+        if variant == "2d3d":
+            a, b, shape, k, fn = rnd(gen, tot8, d1, dtype=dt), rnd(gen, G, d1, d2, dtype=dt, scale=0.1), (tot8, d2), d1, K_.grouped_mm_2d3d
+        elif variant == "3d3d":
+            a, b, shape, k, fn, offs = rnd(gen, G, d2, d1, dtype=dt), rnd(gen, G, d1, 264, dtype=dt, scale=0.1), (G, d2, 264), d1, K_.grouped_mm_3d3d, None
+        elif variant == "2d2d":
+            a, b, shape, k, fn = rnd(gen, d1, tot8, dtype=dt), rnd(gen, tot8, d2, dtype=dt, scale=0.1), (G, d1, d2), max(sizes), K_.grouped_mm_2d2d
+        else:
+            a, b, shape, k, fn = rnd(gen, G, d1, d2, dtype=dt), rnd(gen, d2, tot8, dtype=dt, scale=0.1), (d1, tot8), d2, K_.grouped_mm_3d2d
+        ad, bd = a.to(DEV), b.to(DEV)
+        if a_col:
+            ad = ad.transpose(-2, -1).contiguous().transpose(-2, -1)
+        if b_col:
+            bd = bd.transpose(-2, -1).contiguous().transpose(-2, -1)
+        out = torch.full(shape, float("nan"), device=DEV, dtype=out_dt)
+        what = f"{variant} sizes={sizes} d1={d1} d2={d2} {dt} -> {out_dt} a_col={a_col} b_col={b_col}"
+        with K_.forced_path("mfma"):
+            if offs is None:
+                fn(ad, bd, out)
+            else:
+                fn(ad, bd, offs.to(DEV), out)
+            torch.cuda.synchronize()
+        want = oracle.grouped_mm(a, b, offs, out_dtype=out_dt)
+        got = out.cpu()
+        assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs: " + what
+        oracle.assert_close(got, want, max(k, 1), what=what)
+
+
 # ------------------------------------------------------------------ dtypes
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-4), (torch.float16, 2e-2)])
 def test_fp32_and_fp16_inputs(dtype, tol):
