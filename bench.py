@@ -30,8 +30,8 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the copy-kernel
 # calibration); see profiles/.  None where no profile has been taken.
-MEASURED_TRAFFIC = {"mixtral": 4480476792, "fine": 726500146, "batched": 744756310, "batched_colmajor": None,
-                    "kgrouped": 7105202404, "ngrouped": 1401091215}
+MEASURED_TRAFFIC = {"mixtral": 4328005393, "fine": 689374141, "batched": 671593906, "batched_colmajor": None,
+                    "kgrouped": 7000566520, "ngrouped": 1356381393}
 
 
 def load_sizes(key):
