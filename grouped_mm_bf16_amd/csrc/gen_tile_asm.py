@@ -59,6 +59,9 @@ DBG_COPY_OOB = int(os.environ.get("GMM_GEN_DBG_COPY_OOB", "0"))  # timing only: 
 DBG_NO_READS = int(os.environ.get("GMM_GEN_DBG_NO_READS", "0"))  # timing only: no fragment reads in the loop
 DBG_NO_MASK = int(os.environ.get("GMM_GEN_DBG_NO_MASK", "0"))
 PARTIAL_WAITS = int(os.environ.get("GMM_GEN_PARTIAL_WAITS", "1"))  # MFMAs wait for their own fragments only
+# cache-policy bits of the copies of A and of B ("", "nt", "sc1", "sc0 sc1", "sc1 nt" ...)
+A_POLICY = os.environ.get("GMM_GEN_A_POLICY", "")
+B_POLICY = os.environ.get("GMM_GEN_B_POLICY", "")
 FAST_PATH = int(os.environ.get("GMM_GEN_FAST_PATH", "1"))  # interior K tiles without the per-copy tail / range selects
 DBG_VMCNT = int(os.environ.get("GMM_GEN_DBG_VMCNT", "-1"))  # timing experiments only: copies left in flight at the K-tile barrier
 DBG_TIMING = int(os.environ.get("GMM_GEN_DBG_TIMING", "0"))  # phase timestamps in s[92:99] (extra asm output)
@@ -251,7 +254,9 @@ class Variant:
             out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(vn), vr(vt), sr(s_tail, 2)))
             out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(tmp), vr(V_OOB), sr(s_oob, 2)))
             src = vr(tmp)
-        out.append("buffer_load_dwordx4 %s, %s, %s offen lds" % (src, sr(S_RA if is_a else S_RB, 4), sr(s_ka if is_a else s_kb)))
+        pol = A_POLICY if is_a else B_POLICY
+        out.append("buffer_load_dwordx4 %s, %s, %s offen%s lds" % (src, sr(S_RA if is_a else S_RB, 4), sr(s_ka if is_a else s_kb),
+                                                                  (" " + pol) if pol else ""))
         return out
 
 
