@@ -12,31 +12,41 @@ the pipeline.  Here every register is named, so nothing is spilled and the issue
 order is exactly the one below.
 
 One block computes one 256 x 256 output tile with 4 waves (2 x 2, 128 x 128 per
-wave, 4 x 4 MFMA blocks of 32 x 32):
+wave, 4 x 4 MFMA blocks of 32 x 32); variants for 128 x 256 and 64 x 256 tiles
+(group remainders, small groups), for fp16 instead of bf16 elements, and an
+8-wave form of the 256 x 256 tile (two waves per SIMD, 128 x 64 per wave):
 
   * K is walked in tiles of 64; A and B tiles are copied global -> LDS by
-    buffer_load_dwordx4 ... lds (no registers involved) into two buffers;
+    buffer_load_dwordx4 ... lds (no registers involved) into two buffers (three
+    for the 128- and 64-row tiles, which have the LDS room and need the deeper
+    prefetch);
   * an operand that is contiguous along K lives in LDS as [row][64 k] with its
     16-byte chunks XOR-swizzled (conflict-free ds_read_b128 fragments); one that
     is contiguous along M / N lives as [k][256] in blocks of two k rows with a
     64-byte pad, read with ds_read_b64_tr_b16 (the LDS transposes 4 x 16 blocks);
   * per k16 step a wave issues 16 v_mfma_f32_32x32x16_bf16 and, between them, the
-    8 fragment reads of the next step and its share of the copies of the next
-    tiles, so the matrix pipe never waits on LDS latency;
+    fragment reads of the next step (A block 0, the B blocks, then the other A
+    blocks: each MFMA waits only for its own operands, lgkmcnt counts down in
+    order) and its share of the copies of the next tiles;
+  * the loop body exists twice: K tiles whose copies are neither the last tile of
+    the range nor past it use the copy offsets as they are; the others select
+    per copy between the normal offsets, the last tile's offsets and "out of
+    range" (a buffer load that fetches nothing and writes zeros);
   * one s_barrier per K tile, placed after step 2 so that step 3's MFMAs run
     while the barrier's stragglers arrive and the first fragments of the next
     tile are fetched under them;
-  * epilogue, bf16: the MFMA operands are swapped so a lane owns 4 consecutive
-    columns, packs them (v_cvt_pk_bf16_f32), stages the wave's 128 x 128 block in
-    LDS and writes 16 bytes per lane, 256 contiguous bytes per row;
+  * epilogue, 16-bit output: the MFMA operands are swapped so a lane owns 4
+    consecutive columns, packs them (v_cvt_pk_bf16_f32), stages the wave's block
+    in LDS and writes 16 bytes per lane, 256 contiguous bytes per row; a chunk
+    that a group boundary cuts (jagged columns) goes out as 2-byte stores;
     fp32: each accumulator register goes out as one dword store, 128 contiguous
     bytes per row.
 
-Registers (fixed):
+Registers (4 waves; the 8-wave map is in REGMAPS):
   a[0:255]     accumulators, block (i, j) at a[(4 i + j) 16 ...]
   v[0:15]      A fragments set 0, v[16:31] set 1, v[32:47] B set 0, v[48:63] B set 1
-  v[64:95]     temporaries
-  inputs are pinned by the C++ wrapper to v[128:...] and s[36:...] (see TileRegs).
+  v[64:121]    temporaries, per-buffer fragment addresses of the 3-buffer variants
+  inputs are pinned by the C++ wrapper to v[128:...] and s[28:55] (see GmmTileRegs).
 """
 import os
 import sys
