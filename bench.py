@@ -77,6 +77,14 @@ def make_workload(name, torch):
                  flops=2.0 * 4096 * 16384 * 14336, bound="mfma", k=16384,
                  bytes=a.numel() * 2 + b.numel() * 2 + 8 * 4096 * 14336 * 4,
                  desc="k_grouped_weight_grad_2d2d_G8_M4096_Ktotal16384_N14336_fp32out")
+    elif name == "plain":
+        # the Mixtral workload's FLOPs as ONE group: what the same tile does without any grouping
+        a = torch.randn(1, 16384, 4096, generator=g1).to(bf)
+        b = (torch.randn(1, 4096, 14336, generator=g2) * 0.02).to(bf)
+        w = dict(variant="3d3d", sizes=None, a=a, b=b, out_shape=(1, 16384, 14336), out_dtype=bf,
+                 flops=2.0 * 16384 * 4096 * 14336, bound="mfma", k=4096,
+                 bytes=a.numel() * 2 + b.numel() * 2 + 16384 * 14336 * 2,
+                 desc="plain_gemm_3d3d_G1_M16384_K4096_N14336")
     elif name == "ngrouped":
         sizes = load_sizes("mixtral_top2_g8")
         a = torch.randn(8, 4096, 4096, generator=g1).to(bf)
@@ -152,6 +160,45 @@ def cpu_baseline(w, torch, budget_s=15.0):
             "sample": sample, "seconds": round(t, 3)}
 
 
+def mfma_only(args, torch, dev):
+    """Rate of the matrix pipe alone (register-only loop of the MFMA the kernels use), with operand values
+    drawn like the workload's (N(0,1) for A fragments, 0.02 N(0,1) for B fragments) and with zeros."""
+    import ctypes
+    from grouped_mm_bf16_amd import _lib
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(3)
+    iters = 4000
+    out = torch.empty(512 * 256 * 2, dtype=torch.float32, device=dev)
+    res = {}
+    for label, scale in (("random", 1.0), ("zeros", 0.0)):
+        # fragments alternate: 4 for A (unit scale), 4 for B (0.02), per thread
+        vals = torch.randn(4096, 8, generator=gen) * scale
+        vals[(torch.arange(4096) % 8) >= 4] *= 0.02
+        frags = vals.to(torch.bfloat16).to(dev)
+        for waves in (1, 2):
+            blocks = ctypes.c_int32(0)
+
+            def launch():
+                _lib.check(lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), out.numel() * 4,
+                                                  waves, iters, ctypes.addressof(blocks),
+                                                  torch.cuda.current_stream().cuda_stream), "gmm_diag_mfma_rate")
+            for _ in range(args.warmup):
+                launch()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(args.steps):
+                launch()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / args.steps
+            flops = blocks.value * 4 * iters * 16 * 32768.0
+            res[f"{label}_{waves}_waves_per_simd"] = round(flops / ms / 1e9, 1)
+    print(json.dumps({"metric": "v_mfma_f32_32x32x16_bf16 alone, register operands (context for the MFMA roofline)",
+                      "value": res["random_1_waves_per_simd"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+                      "warmup": args.warmup, "peak": PEAK_BF16_TFLOPS, "detail": res}))
+
+
 def library_comparator(w, a, b, offs, torch, steps):
     """PyTorch-ROCm's own grouped GEMM on the same device tensors: context for `value`, never an oracle."""
     import torch.nn.functional as F
@@ -181,7 +228,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="mixtral",
-                    choices=["mixtral", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "copy"])
+                    choices=["mixtral", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "plain",
+                             "copy", "mfma_only"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--library-comparator", action="store_true",
                     help="also time PyTorch-ROCm's own torch.nn.functional.grouped_mm on the same tensors (context only)")
@@ -214,6 +262,9 @@ def main():
         print(json.dumps({"metric": "device copy of 1 GiB (calibration)", "value": round(2 * (1 << 30) / ms / 1e6, 1),
                           "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
                           "ms_per_step": round(ms, 4), "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
+        return
+    if args.workload == "mfma_only":
+        mfma_only(args, torch, dev)
         return
     w = make_workload(args.workload, torch)
     a, b = w["a"].to(dev), w["b"].to(dev)

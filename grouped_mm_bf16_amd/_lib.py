@@ -37,6 +37,7 @@ SIGNATURES = {
     "gmm_host_tile_list": (_i64, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _i64]),
     "gmm_host_tile_list2": (_i64, [_vp] + [_i32] * 11 + [_vp, _i64]),
     "gmm_set_tile_heights": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
+    "gmm_diag_mfma_rate": (ctypes.c_int, [_vp, _i64, _vp, _i64, _i32, _i32, _vp, _vp]),
 }
 
 _lock = threading.Lock()

@@ -123,6 +123,15 @@ int64_t gmm_host_tile_list2(const int32_t* offs_host, int32_t G, int32_t jagged,
                             int32_t xcd_remap, int32_t num_workgroups,
                             int32_t* records, int64_t capacity);
 
+/* Diagnostic, no counterpart in the reference: launches a register-only loop of independent
+ * v_mfma_f32_32x32x16_bf16 on every SIMD (waves_per_simd 1 or 2; 16 MFMAs of 32768 FLOP per wave and
+ * iteration), with operand fragments taken from `frags` (device memory, frag_bytes >= 16, bf16 values of
+ * the caller's choice: the sustained clock depends on them).  `out` receives one float per thread
+ * (blocks * 256 floats); *blocks gets the number of 256-thread blocks launched, so that
+ * FLOP per launch = *blocks * 4 * iters * 16 * 32768.  Returns a gmm_status. */
+int gmm_diag_mfma_rate(const void* frags, int64_t frag_bytes, void* out, int64_t out_bytes,
+                       int32_t waves_per_simd, int32_t iters, int32_t* blocks, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -310,6 +310,23 @@ def test_row_major_and_column_major_b_agree_bit_for_bit():
     assert torch.equal(grouped_mm(a, b).view(torch.int16), grouped_mm(a, b_col).view(torch.int16))
 
 
+def test_mfma_rate_diagnostic_runs():
+    """The register-only MFMA loop behind `bench.py --workload mfma_only`: argument checks and one launch."""
+    import ctypes
+    lib = K_._lib.load()
+    frags = torch.randn(64, 8).to(torch.bfloat16).to(DEV)
+    out = torch.full((512 * 256 * 2,), float("nan"), device=DEV)
+    blocks = ctypes.c_int32(0)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.gmm_diag_mfma_rate(None, 16, out.data_ptr(), out.numel() * 4, 1, 10, ctypes.addressof(blocks), stream) != 0
+    assert lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), 16, 1, 10, ctypes.addressof(blocks), stream) != 0
+    assert lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), out.numel() * 4, 2, 10,
+                                  ctypes.addressof(blocks), stream) == 0
+    torch.cuda.synchronize()
+    n = blocks.value * 256
+    assert blocks.value > 0 and torch.isfinite(out[:n]).all() and torch.isnan(out[n:]).all()
+
+
 # ------------------------------------------------------------------ seeded random sweep
 def _random_case(rng):
     variant = ["2d3d", "3d3d", "2d2d", "3d2d"][int(rng.integers(0, 4))]
