@@ -327,6 +327,47 @@ def test_mfma_rate_diagnostic_runs():
     assert blocks.value > 0 and torch.isfinite(out[:n]).all() and torch.isnan(out[n:]).all()
 
 
+@pytest.mark.parametrize("a_col", [False, True])
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("variant", ["2d3d", "3d3d", "2d2d", "3d2d"])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-4), (torch.bfloat16, None)])
+def test_generic_family_on_the_matrix_cores(variant, a_col, b_col, dtype, tol):
+    """Problems with at least one 128 x 128 tile that the 16-bit MFMA tile does not take (fp32 operands;
+    bf16 with odd extents): the stride-generic kernel built on v_mfma_f32_32x32x2_f32."""
+    gen = torch.Generator().manual_seed(53)
+    sizes = [77, 0, 1, 331, 64, 200]  # sum 673
+    offs = offs_of(sizes)
+    G = len(sizes)
+    if variant == "2d3d":
+        a, b, shape, k, fn = rnd(gen, 673, 203, dtype=dtype), rnd(gen, G, 203, 261, dtype=dtype, scale=0.1), (673, 261), 203, K_.grouped_mm_2d3d
+    elif variant == "3d3d":
+        a, b, shape, k, fn, offs = rnd(gen, 3, 301, 203, dtype=dtype), rnd(gen, 3, 203, 261, dtype=dtype, scale=0.1), (3, 301, 261), 203, K_.grouped_mm_3d3d, None
+    elif variant == "2d2d":
+        a, b, shape, k, fn = rnd(gen, 261, 673, dtype=dtype), rnd(gen, 673, 269, dtype=dtype, scale=0.1), (G, 261, 269), 331, K_.grouped_mm_2d2d
+    else:
+        a, b, shape, k, fn = rnd(gen, G, 261, 203, dtype=dtype), rnd(gen, 203, 673, dtype=dtype, scale=0.1), (261, 673), 203, K_.grouped_mm_3d2d
+    ad, bd = a.to(DEV), b.to(DEV)
+    if a_col:
+        ad = ad.transpose(-2, -1).contiguous().transpose(-2, -1)
+    if b_col:
+        bd = bd.transpose(-2, -1).contiguous().transpose(-2, -1)
+    out = torch.full(shape, float("nan"), device=DEV, dtype=dtype)
+    if offs is None:
+        fn(ad, bd, out)
+    else:
+        fn(ad, bd, offs.to(DEV), out)
+    torch.cuda.synchronize()
+    assert K_.last_path() == "generic"
+    want = oracle.grouped_mm(a, b, offs, out_dtype=dtype)
+    got = out.cpu()
+    assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs"
+    if tol is None:
+        oracle.assert_close(got, want, k)
+    else:
+        owned = ~torch.isnan(want)
+        torch.testing.assert_close(got[owned], want[owned], rtol=tol, atol=tol)
+
+
 # ------------------------------------------------------------------ seeded random sweep
 def _random_case(rng):
     variant = ["2d3d", "3d3d", "2d2d", "3d2d"][int(rng.integers(0, 4))]
