@@ -28,10 +28,23 @@ if ROOT not in sys.path:
 METRIC = "TFLOP/s + % bf16 MFMA peak, 2D×3D MoE G=8 K=4096 N=14336, 1 GPU"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the copy-kernel
-# calibration); see profiles/.  None where no profile has been taken.
-MEASURED_TRAFFIC = {"mixtral": 4328005393, "fine": 689374141, "batched": 671593906, "batched_colmajor": None,
-                    "kgrouped": 7000566520, "ngrouped": 1356381393}
+# workload -> tag in the name of its rocprofv3 summary under profiles/ (`..__<tag>.md`)
+PROFILE_TAG = {"readme": "readme_2d3d", "mixtral": "mixtral_2d3d", "fine": "fine_grained_2d3d", "batched": "batched_3d3d",
+               "batched_colmajor": "batched_colmajor_3d3d", "kgrouped": "kgrouped_2d2d", "ngrouped": "ngrouped_3d2d"}
+
+
+def measured_traffic(name):
+    """HBM-side bytes per launch of the workload's kernel as its committed rocprofv3 summary states them
+    (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration): the line
+    `traffic_bytes_per_launch: N` of profiles/*__<tag>.md.  Returns (bytes or None, file or None)."""
+    import glob
+    import re
+    tag = PROFILE_TAG.get(name)
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", f"*__{tag}.md"))) if tag else []:
+        m = re.search(r"traffic_bytes_per_launch:\s*(\d+)", open(path).read())
+        if m:
+            return int(m.group(1)), os.path.relpath(path, ROOT)
+    return None, None
 
 
 def load_sizes(key):
@@ -44,7 +57,16 @@ def make_workload(name, torch):
     from grouped_mm_bf16_amd import kernels
     g1, g2 = torch.Generator().manual_seed(1), torch.Generator().manual_seed(2)
     bf = torch.bfloat16
-    if name == "mixtral":
+    if name == "readme":
+        sizes = [0, 7, 1, 13, 0, 11]
+        g0 = torch.Generator().manual_seed(0)
+        a = torch.randn(32, 64, generator=g0).to(bf)
+        b = torch.randn(6, 64, 48, generator=g0).to(bf)
+        w = dict(variant="2d3d", sizes=sizes, a=a, b=b, out_shape=(32, 48), out_dtype=bf,
+                 flops=2.0 * 32 * 64 * 48, bound="latency", k=64,
+                 bytes=a.numel() * 2 + 4 * 64 * 48 * 2 + 32 * 48 * 2,
+                 desc="readme_2d3d_G6_M32_K64_N48_two_empty_groups")
+    elif name == "mixtral":
         sizes = load_sizes("mixtral_top2_g8")
         a = torch.randn(16384, 4096, generator=g1).to(bf)
         b = (torch.randn(8, 4096, 14336, generator=g2) * 0.02).to(bf)
@@ -147,20 +169,42 @@ def cpu_baseline(w, torch, budget_s=15.0):
         sample = (f"groups {sorted(chosen)} of {len(sizes)} ({fl / w['flops'] * 100:.0f}% of the step's FLOPs), "
                   f"median of {len(runs)} timed run(s) after a probe")
     else:
-        # batched / K-grouped: a slab of the first group
-        if w["variant"] == "3d3d":
-            x, y = a[0].float(), b[0].float()
-        elif w["variant"] == "3d2d":
-            x, y = a[0].float(), b[:, :sizes[0]].float()
-        else:
-            e = sizes[0]
-            x, y = a[:, :e].float(), b[:e].float()
-        torch.matmul(x[:64], y)
+        # batched / K-grouped / N-grouped: the groups' own products (3D x 3D: the first batches), as many
+        # as fit about a third of the budget per run; 1 warm-up + 3 timed runs, median
+        G = a.shape[0] if w["variant"] == "3d3d" else len(sizes)
+        ranges = oracle.group_ranges(torch.tensor(sizes).cumsum(0).tolist()) if sizes else None
+
+        def operands(g):
+            if w["variant"] == "3d3d":
+                return a[g].float(), b[g].float()
+            s_, e_ = ranges[g]
+            if w["variant"] == "3d2d":
+                return a[g].float(), b[:, s_:e_].float()
+            return a[:, s_:e_].float(), b[s_:e_].float()
+
+        x, y = operands(0)
+        torch.matmul(x[:64], y)                       # thread-pool start-up
         t0 = time.perf_counter()
-        torch.matmul(x, y)
-        t = time.perf_counter() - t0
-        fl = 2.0 * x.shape[0] * x.shape[1] * y.shape[1]
-        sample = f"first group only ({fl / w['flops'] * 100:.0f}% of the step's FLOPs), 1 timed run"
+        torch.matmul(x, y)                            # warm-up run = the probe
+        rate = 2.0 * x.shape[0] * x.shape[1] * y.shape[1] / max(time.perf_counter() - t0, 1e-9)
+        chosen, ops, work = [], [], 0.0
+        for g in range(G):
+            x, y = operands(g)
+            f = 2.0 * x.shape[0] * x.shape[1] * y.shape[1]
+            if f == 0 or (chosen and (work + f) / rate > budget_s / 3):
+                continue
+            chosen.append(g)
+            ops.append((x, y))
+            work += f
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for x, y in ops:
+                torch.matmul(x, y)
+            times.append(time.perf_counter() - t0)
+        t, fl = sorted(times)[1], work
+        sample = (f"groups {chosen} of {G} ({fl / w['flops'] * 100:.0f}% of the step's FLOPs), "
+                  f"median of 3 timed runs after a warm-up")
     return {"value": round(fl / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "sample": sample, "seconds": round(t, 3)}
 
@@ -227,15 +271,111 @@ def library_comparator(w, a, b, offs, torch, steps):
             "unit": "TFLOP/s", "ms_per_step": round(ms, 4)}
 
 
+def parity_check(w, out, offs, torch, oracle):
+    """Oracle comparison on the tensors that are about to be timed: the whole output of the small README
+    case, otherwise a sample of rows of the first, a middle and the last group (K per element's own group)."""
+    got = out.cpu()
+    a, b = w["a"], w["b"]
+    if w["desc"].startswith("readme"):
+        oracle.assert_close(got, oracle.grouped_mm(a, b, offs.cpu()), w["k"], what="bench parity")
+        return
+    ranges = oracle.group_ranges(offs.cpu().tolist()) if offs is not None else None
+    G = a.shape[0] if w["variant"] == "3d3d" else len(ranges)
+    for g in sorted({0, G // 2, G - 1}):
+        if w["variant"] == "2d3d":
+            s_, e_ = ranges[g]
+            if e_ == s_:
+                continue
+            rows = sorted({s_, (s_ + e_) // 2, e_ - 1})
+            want = (a[rows].float() @ b[g].float()).to(got.dtype)
+            oracle.assert_close(got[rows], want, w["k"], what=f"bench parity rows {rows} group {g}")
+        elif w["variant"] == "3d3d":
+            rows = [0, a.shape[1] // 2, a.shape[1] - 1]
+            want = (a[g][rows].float() @ b[g].float()).to(got.dtype)
+            oracle.assert_close(got[g][rows], want, w["k"], what=f"bench parity batch {g}")
+        elif w["variant"] == "2d2d":
+            s_, e_ = ranges[g]
+            rows = [0, a.shape[0] // 2, a.shape[0] - 1]
+            want = (a[rows][:, s_:e_].float() @ b[s_:e_].float()).to(got.dtype)
+            oracle.assert_close(got[g][rows], want, e_ - s_, what=f"bench parity group {g}")
+        else:
+            s_, e_ = ranges[g]
+            rows = [0, a.shape[1] // 2, a.shape[1] - 1]
+            want = (a[g][rows].float() @ b[:, s_:e_].float()).to(got.dtype)
+            oracle.assert_close(got[rows][:, s_:e_], want, w["k"], what=f"bench parity group {g}")
+
+
+def run_workload(name, steps, warmup, torch, dev, path="auto", wall=True):
+    """Times one workload on tensors resident in HBM.  Returns (w, record): `record` has the wall-clock time
+    over exactly `steps` steps (when `wall`), the per-launch kernel times from HIP events on the launch
+    stream, the roofline position and a parity flag."""
+    from grouped_mm_bf16_amd import kernels
+    from oracle import grouped_mm_oracle as oracle
+    w = make_workload(name, torch)
+    a, b = w["a"].to(dev), w["b"].to(dev)
+    if w.get("b_col"):
+        b = b.transpose(-2, -1).contiguous().transpose(-2, -1)
+    offs = None
+    if w["sizes"] is not None:
+        offs = torch.tensor(w["sizes"], dtype=torch.int64).cumsum(0).to(torch.int32).to(dev)
+    out = torch.empty(w["out_shape"], device=dev, dtype=w["out_dtype"])
+
+    def step():
+        if offs is None:
+            w["launch"](a, b, out)
+        else:
+            w["launch"](a, b, offs, out)
+
+    with kernels.forced_path(path):
+        step()
+        torch.cuda.synchronize()
+        parity_check(w, out, offs, torch, oracle)        # raises on a mismatch: nothing wrong gets timed
+        family = kernels.last_path()
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        ms_per_step = None
+        if wall:
+            # whole-job wall clock over exactly `steps` steps
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+        # per-launch kernel time: HIP events on the launch stream around each step
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for e0, e1 in evs:
+            e0.record()
+            step()
+            e1.record()
+        torch.cuda.synchronize()
+        k_ms = [e0.elapsed_time(e1) for e0, e1 in evs]
+    k_avg = statistics.mean(k_ms)
+    if w["bound"] == "hbm":
+        achieved, peak, unit = w["bytes"] / (k_avg * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+    else:
+        achieved, peak, unit = w["flops"] / (k_avg * 1e-3) / 1e12, PEAK_BF16_TFLOPS, "TFLOP/s"
+    traffic, source = measured_traffic(name)
+    roof = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": traffic, "traffic_source": source,
+            "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(k_ms), 4),
+            "kernel_ms_median": round(statistics.median(k_ms), 4),
+            "algorithmic_flops": w["flops"], "algorithmic_bytes": w["bytes"]}
+    del a, b, out
+    return w, {"ms_per_step": ms_per_step, "family": family, "roofline": roof, "parity": "ok"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="mixtral",
-                    choices=["mixtral", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "plain",
+                    choices=["mixtral", "readme", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "plain",
                              "copy", "mfma_only"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the short runs of the other BASELINE configurations (the `configs` object)")
     ap.add_argument("--library-comparator", action="store_true",
                     help="also time PyTorch-ROCm's own torch.nn.functional.grouped_mm on the same tensors (context only)")
     ap.add_argument("--path", default="auto", choices=["auto", "mfma", "generic"])
@@ -247,8 +387,6 @@ def main():
     import torch
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
-    from grouped_mm_bf16_amd import kernels
-    from oracle import grouped_mm_oracle as oracle
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -271,76 +409,44 @@ def main():
     if args.workload == "mfma_only":
         mfma_only(args, torch, dev)
         return
-    w = make_workload(args.workload, torch)
-    a, b = w["a"].to(dev), w["b"].to(dev)
-    if w.get("b_col"):
-        b = b.transpose(-2, -1).contiguous().transpose(-2, -1)
-    offs = None
-    if w["sizes"] is not None:
-        offs = torch.tensor(w["sizes"], dtype=torch.int64).cumsum(0).to(torch.int32).to(dev)
-    out = torch.empty(w["out_shape"], device=dev, dtype=w["out_dtype"])
 
-    def step():
-        if offs is None:
-            w["launch"](a, b, out)
-        else:
-            w["launch"](a, b, offs, out)
-
-    with kernels.forced_path(args.path):
-        # parity spot-check on the tensors that are about to be timed
-        step()
-        torch.cuda.synchronize()
-        if w["variant"] == "2d3d":
-            ol = offs.cpu().tolist()
-            for r in (0, ol[0] - 1 if ol[0] > 0 else 0, ol[-1] - 1):
-                g = oracle.upper_bound(ol, r)
-                want = (w["a"][r:r + 1].float() @ w["b"][g].float()).to(out.dtype)
-                oracle.assert_close(out[r:r + 1].cpu(), want, w["k"], what=f"bench parity row {r}")
-        path = kernels.last_path()
-
-        for _ in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        # whole-job wall clock over exactly `steps` steps
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        # per-launch kernel time: HIP events on the launch stream around each step
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-               for _ in range(args.steps)]
-        for e0, e1 in evs:
-            e0.record()
-            step()
-            e1.record()
-        torch.cuda.synchronize()
-        k_ms = [e0.elapsed_time(e1) for e0, e1 in evs]
-
-    ms_per_step = wall / args.steps * 1e3
-    tflops = w["flops"] / (ms_per_step * 1e-3) / 1e12
-    k_avg = statistics.mean(k_ms)
-    if w["bound"] == "mfma":
-        achieved, peak, unit = w["flops"] / (k_avg * 1e-3) / 1e12, PEAK_BF16_TFLOPS, "TFLOP/s"
-    else:
-        achieved, peak, unit = w["bytes"] / (k_avg * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+    w, r = run_workload(args.workload, args.steps, args.warmup, torch, dev, args.path)
+    tflops = w["flops"] / (r["ms_per_step"] * 1e-3) / 1e12
     rec = {
         "metric": METRIC, "value": round(tflops, 2), "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(r["ms_per_step"], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": w["desc"], "kernel_family": path,
+        "config": {"workload": w["desc"], "kernel_family": r["family"],
                    "pct_bf16_mfma_peak": round(tflops / PEAK_BF16_TFLOPS * 100, 2)},
-        "roofline": {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
-                     "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(k_ms), 4),
-                     "kernel_ms_median": round(statistics.median(k_ms), 4),
-                     "algorithmic_flops": w["flops"], "algorithmic_bytes": w["bytes"]},
+        "roofline": r["roofline"],
     }
     if args.library_comparator:
+        # same tensors again (the workload's own were freed with its run)
+        a, b = w["a"].to(dev), w["b"].to(dev)
+        offs = None if w["sizes"] is None else torch.tensor(w["sizes"]).cumsum(0).to(torch.int32).to(dev)
         rec["library_comparator"] = library_comparator(w, a, b, offs, torch, args.steps)
+        del a, b
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(w, torch)
+    del w
+    if args.workload == "mixtral" and not args.no_configs:
+        # The other BASELINE configurations, a few steps each (kernel time from HIP events; the headline
+        # fields above are the Mixtral workload's alone).
+        rec["configs"] = {}
+        for name in ("readme", "batched", "batched_colmajor", "fine", "kgrouped"):
+            try:
+                wi, ri = run_workload(name, 10, 3, torch, dev, args.path, wall=False)
+                k_avg = ri["roofline"]["kernel_ms_avg"]
+                rec["configs"][name] = {
+                    "workload": wi["desc"], "kernel_family": ri["family"], "ms": k_avg,
+                    "tflops": round(wi["flops"] / (k_avg * 1e-3) / 1e12, 2),
+                    "gbs": round(wi["bytes"] / (k_avg * 1e-3) / 1e9, 1),
+                    "bound": wi["bound"], "frac": ri["roofline"]["frac"] if wi["bound"] != "latency" else None,
+                    "traffic": ri["roofline"]["traffic"], "parity": ri["parity"], "steps": 10}
+                del wi
+            except Exception as ex:   # a config that fails must not take the headline down with it
+                rec["configs"][name] = {"parity": "FAILED", "error": repr(ex)[:300]}
     print(json.dumps(rec))
 
 

@@ -13,8 +13,7 @@ order is exactly the one below.
 
 One block computes one 256 x 256 output tile with 4 waves (2 x 2, 128 x 128 per
 wave, 4 x 4 MFMA blocks of 32 x 32); variants for 128 x 256 and 64 x 256 tiles
-(group remainders, small groups), for fp16 instead of bf16 elements, and an
-8-wave form of the 256 x 256 tile (two waves per SIMD, 128 x 64 per wave):
+(group remainders, small groups) and for fp16 instead of bf16 elements:
 
   * K is walked in tiles of 64; A and B tiles are copied global -> LDS by
     buffer_load_dwordx4 ... lds (no registers involved) into two buffers (three
@@ -42,79 +41,43 @@ wave, 4 x 4 MFMA blocks of 32 x 32); variants for 128 x 256 and 64 x 256 tiles
     fp32: each accumulator register goes out as one dword store, 128 contiguous
     bytes per row.
 
-Registers (4 waves; the 8-wave map is in REGMAPS):
+Registers:
   a[0:255]     accumulators, block (i, j) at a[(4 i + j) 16 ...]
   v[0:15]      A fragments set 0, v[16:31] set 1, v[32:47] B set 0, v[48:63] B set 1
   v[64:121]    temporaries, per-buffer fragment addresses of the 3-buffer variants
   inputs are pinned by the C++ wrapper to v[128:...] and s[28:55] (see GmmTileRegs).
 """
-import os
 import sys
 
 # copies (of the 16 per K tile and wave) issued in: step 3 right after the barrier, then steps 0, 1, 2
 # of the next K tile; the tile must have landed at that tile's barrier (end of its step 2).
-COPY_SCHEDULE = tuple(int(x) for x in os.environ.get("GMM_GEN_COPY_SCHEDULE", "8,8,0,0").split(","))
-assert len(COPY_SCHEDULE) == 4 and sum(COPY_SCHEDULE) == 16
-COPY_SCHEDULE8 = tuple(int(x) for x in os.environ.get("GMM_GEN_COPY_SCHEDULE8", "4,4,0,0").split(","))  # 8 waves: 8 copies
-assert len(COPY_SCHEDULE8) == 4 and sum(COPY_SCHEDULE8) == 8
-
-# L2 prefetch distance in K tiles (0 = off): in step 2 of K tile kt every lane touches one cache line of
-# K tile kt + PREFETCH of each operand, so that the copies issued two tiles later hit in L2.
-PREFETCH = int(os.environ.get("GMM_GEN_PREFETCH", "0"))
-
-# timing experiments only (results are wrong with these on)
-DBG_NO_COPY = int(os.environ.get("GMM_GEN_DBG_NO_COPY", "0"))
-DBG_NO_BARRIER = int(os.environ.get("GMM_GEN_DBG_NO_BARRIER", "0"))
-DBG_COPY_OOB = int(os.environ.get("GMM_GEN_DBG_COPY_OOB", "0"))  # timing only: loop copies fetch nothing (write zeros)
-DBG_NO_READS = int(os.environ.get("GMM_GEN_DBG_NO_READS", "0"))  # timing only: no fragment reads in the loop
-DBG_NO_MASK = int(os.environ.get("GMM_GEN_DBG_NO_MASK", "0"))
-PARTIAL_WAITS = int(os.environ.get("GMM_GEN_PARTIAL_WAITS", "1"))  # MFMAs wait for their own fragments only
-# cache-policy bits of the copies of A and of B ("", "nt", "sc1", "sc0 sc1", "sc1 nt" ...)
-A_POLICY = os.environ.get("GMM_GEN_A_POLICY", "")
-B_POLICY = os.environ.get("GMM_GEN_B_POLICY", "")
-FAST_PATH = int(os.environ.get("GMM_GEN_FAST_PATH", "1"))  # interior K tiles without the per-copy tail / range selects
-DBG_VMCNT = int(os.environ.get("GMM_GEN_DBG_VMCNT", "-1"))  # timing experiments only: copies left in flight at the K-tile barrier
-DBG_TIMING = int(os.environ.get("GMM_GEN_DBG_TIMING", "0"))  # phase timestamps in s[92:99] (extra asm output)
+COPY_SCHEDULE = (8, 8, 0, 0)
 
 PITCH = 272           # bytes per staged row of 128 bf16 (256 + 16: shifts banks per row)
 TR_BLOCK = 1088       # two k rows of 512 bytes + 64 bytes pad
 KC_STAGE = 256 * 64 * 2
 TR_STAGE = 32 * TR_BLOCK
+# 256-row tile: K is walked in half tiles of 32 through a ring of four LDS slots per operand
+RING = 4
+RING_ENABLED = False
+RING_KC_SLOT = 256 * 32 * 2      # [row][32 k]: 64-byte rows, chunks XOR-swizzled by (row >> 2) & 3
+RING_TR_SLOT = 16 * TR_BLOCK     # [k][256] in 16 blocks of two k rows
 STAGE_BYTES = 4 * 128 * PITCH
 
-# ---- fixed register maps ---------------------------------------------------
-# 4 waves (one per SIMD, 128 x 128 per wave, 256 accumulators): the wave owns all 512 registers of a lane.
-# 8 waves (two per SIMD, 128 x 64 per wave, 128 accumulators): 128 + 128 registers per wave.
-STAGES_SHORT = int(os.environ.get('GMM_GEN_STAGES_SHORT', '3'))  # LDS buffers of the 128- and 64-row tiles
-REGMAPS = {
-    4: dict(V_AF=[0, 16],        # A fragment sets (4 x 4 registers each)
-            V_BF=[32, 48],
-            V_TMP=64,            # 64..95
-            V_VOA_HEAD=128, V_VOB_HEAD=136, V_VOA=144, V_VOB=152, V_VOA_TAIL=160, V_VOB_TAIL=168,
-            V_RA=176, V_RB=180,  # fragment read addresses (4 + 4)
-            V_EPI=184,           # +0: stage write addr, +1: stage read addr, +2: store voffset, +3: row - row_lo
-            V_OOB=188,           # constant 0x80000000
-            V_EPI2=190,          # +0: store voffset whatever the chunk's validity, +1: mask of valid elements if partial
-            V_PF=192,            # A / B prefetch offsets
-            V_PFD=96,            # dummy destinations of the prefetch loads (96, 97)
-            V_BUFA=98, V_BUFB=110,  # three-buffer variants: fragment addresses per (buffer, step), 12 + 12
-            V_FIX=196,           # A first-chunk addr, A last-chunk addr, same for B (buffer 0)
-            V_CLOBBER=122),
-    8: dict(V_AF=[0, 24],        # A 4 x 4 registers, B 2 x 4 registers per set
-            V_BF=[16, 40],
-            V_TMP=48,            # 48..79
-            V_VOA_HEAD=80, V_VOB_HEAD=84, V_VOA=88, V_VOB=92, V_VOA_TAIL=96, V_VOB_TAIL=100,
-            V_RA=104, V_RB=108, V_EPI=112, V_FIX=116, V_OOB=120,
-            V_PF=None, V_PFD=None, V_BUFA=None, V_BUFB=None, V_EPI2=None,
-            V_CLOBBER=80),
-}
-
-
-def use_regmap(waves):
-    globals().update(REGMAPS[waves])
-
-
-use_regmap(4)
+# ---- fixed register map: one wave per SIMD (128 x 128 per wave, 256 accumulators), the wave owns all 512
+# registers of a lane.
+STAGES_SHORT = 3         # LDS buffers of the 128- and 64-row tiles
+V_AF = [0, 16]           # A fragment sets (4 x 4 registers each)
+V_BF = [32, 48]
+V_TMP = 64               # 64..95
+V_VOA_HEAD, V_VOB_HEAD, V_VOA, V_VOB, V_VOA_TAIL, V_VOB_TAIL = 128, 136, 144, 152, 160, 168
+V_RA, V_RB = 176, 180    # fragment read addresses (4 + 4)
+V_EPI = 184              # +0: stage write addr, +1: stage read addr, +2: store voffset, +3: row - row_lo
+V_OOB = 188              # constant 0x80000000
+V_EPI2 = 190             # +0: store voffset whatever the chunk's validity, +1: mask of valid elements if partial
+V_BUFA, V_BUFB = 98, 110  # three-buffer variants: fragment addresses per (buffer, step), 12 + 12
+V_FIX = 196              # A first-chunk addr, A last-chunk addr, same for B (buffer 0)
+V_CLOBBER = 122
 S_MASK = 28            # s[28:31] keep-mask of the first chunk of the k range, s[32:35] of the last chunk
 
 S_RA, S_RB, S_RC = 36, 40, 44   # buffer resources
@@ -137,9 +100,6 @@ class Emit:
         return "\n".join('      "%s\\n\\t"' % l for l in self.lines)
 
 
-PITCH8 = 144          # 8 waves: bytes per staged row of 64 bf16 (128 + 16)
-
-
 def vr(base, n=1):
     return "v%d" % base if n == 1 else "v[%d:%d]" % (base, base + n - 1)
 
@@ -151,25 +111,32 @@ def sr(base, n=1):
 class Variant:
     """tm = MFMA block rows per wave: the tile is 64 tm rows (256 / 128 / 64) by 256 columns."""
 
-    def __init__(self, a_tr, b_tr, out_f32, tm=4, waves=4, f16=0):
-        self.a_tr, self.b_tr, self.out_f32, self.tm, self.waves, self.f16 = a_tr, b_tr, out_f32, tm, waves, f16
+    def __init__(self, a_tr, b_tr, out_f32, tm=4, f16=0):
+        self.a_tr, self.b_tr, self.out_f32, self.tm, self.f16 = a_tr, b_tr, out_f32, tm, f16
         self.dt = "f16" if f16 else "bf16"   # element type of A, B and of a 16-bit output
-        assert tm in (1, 2, 4) and (tm == 4 or not a_tr) and (waves == 4 or (waves == 8 and tm == 4 and not PREFETCH))
-        self.tn = 16 // waves            # 32-column MFMA blocks per wave (the wave grid is 2 x waves / 2)
-        self.na = 8 * tm // waves        # copies of the A tile per wave and K tile
-        self.nb = 32 // waves            # ... of the B tile
+        assert tm in (1, 2, 4) and (tm == 4 or not a_tr)
+        self.tn = 4                      # 32-column MFMA blocks per wave (the wave grid is 2 x 2)
+        self.na = 2 * tm                 # copies of the A tile per wave and K tile
+        self.nb = 8                      # ... of the B tile
         self.ncopy = self.na + self.nb
         c3 = (self.ncopy + 1) // 2
-        self.sched = COPY_SCHEDULE if (tm == 4 and waves == 4) else COPY_SCHEDULE8 if waves == 8 else (c3, self.ncopy - c3, 0, 0)
+        self.sched = COPY_SCHEDULE if tm == 4 else (c3, self.ncopy - c3, 0, 0)
         # LDS buffers per operand: 2 for the 256-row tile (LDS is full), 3 for the shorter ones, whose K
         # tiles are short of MFMA work and would otherwise wait on memory latency every K tile
         self.stages = STAGES_SHORT if tm < 4 else 2
         self.a_stage = TR_STAGE if a_tr else (64 * tm * 128 if self.stages == 3 else KC_STAGE)
         self.b_stage = TR_STAGE if b_tr else KC_STAGE
         self.b_base = self.stages * self.a_stage   # LDS offset of B buffer 0
+        self.ring = RING_ENABLED and tm == 4
+        if self.ring:
+            self.na = self.nb = 4                # copies per wave and half tile, per operand
+            self.ncopy = 8
+            self.stages = RING
+            self.a_stage = RING_TR_SLOT if a_tr else RING_KC_SLOT
+            self.b_stage = RING_TR_SLOT if b_tr else RING_KC_SLOT
+            self.b_base = RING * self.a_stage
         self.swap = not out_f32                  # bf16: lanes own 4 consecutive columns
-        self.name = "%s%s_%s_%s_m%d%s" % ("t" if a_tr else "k", "t" if b_tr else "k", self.dt, "f32" if out_f32 else self.dt,
-                                          64 * tm, "_w8" if waves == 8 else "")
+        self.name = "%s%s_%s_%s_m%d" % ("t" if a_tr else "k", "t" if b_tr else "k", self.dt, "f32" if out_f32 else self.dt, 64 * tm)
 
     def acc(self, i, j):
         return (self.tn * i + j) * 16
@@ -185,17 +152,20 @@ class Variant:
         ):
             # two buffers: the buffer is an immediate offset; three: one address register per buffer and
             # step (set up by the prologue), because the offsets no longer fit the 16-bit immediate
-            if self.stages == 2:
+            if self.stages == 2 or self.ring:
                 reg, boff = (vaddr + s if not tr else vaddr), buf * stage
             else:
                 reg, boff = (vbuf + 4 * buf + s if not tr else vbuf + 4 * buf), 0
+            sub = 2048 if self.ring else 4096
             for x in range(nblk):
                 d = vbase + 4 * x
                 if not tr:
-                    # address register per step; sub-tiles are 32 rows = 4096 bytes apart
-                    blocks[(op, x)] = ["ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(reg), boff + x * 4096)]
+                    # address register per step; sub-tiles are 32 rows = 4096 bytes apart (2048 in the ring's 64-byte rows)
+                    assert boff + x * sub < 65536
+                    blocks[(op, x)] = ["ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(reg), boff + x * sub)]
                 else:
                     o = boff + s * 8 * TR_BLOCK + x * 64
+                    assert o + 512 < 65536
                     blocks[(op, x)] = ["ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d, 2), vr(reg), o),
                                        "ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d + 2, 2), vr(reg), o + 512)]
         self.read_order = [("A", 0)] + [("B", x) for x in range(self.tn)] + [("A", x) for x in range(1, self.tm)]
@@ -235,8 +205,9 @@ class Variant:
     # s_ka / s_kb: SGPRs with the tile's byte offsets along K for A and B.  which: "head" or "loop".
     def dma(self, n, buf, which, s_tail, s_oob, s_ka, s_kb, tmp):
         out = []
-        is_a = n < self.na
-        i = n if is_a else n - self.na
+        # ring: B's copies go first (B is the operand that streams from HBM in the MoE shapes)
+        is_a = n >= self.nb if self.ring else n < self.na
+        i = (n - self.nb if is_a else n) if self.ring else (n if is_a else n - self.na)
         tr = self.a_tr if is_a else self.b_tr
         stage = self.a_stage if is_a else self.b_stage
         lbase = 0 if is_a else self.b_base
@@ -252,11 +223,7 @@ class Variant:
         if which == "head":
             vo = (V_VOA_HEAD if is_a else V_VOB_HEAD) + i
             src = vr(vo)
-        elif DBG_NO_COPY:
-            return []
-        elif DBG_COPY_OOB:
-            src = vr(V_OOB)
-        elif DBG_NO_MASK or which == "fast":
+        elif which == "fast":
             src = vr((V_VOA if is_a else V_VOB) + i)
         else:
             vn = (V_VOA if is_a else V_VOB) + i
@@ -264,9 +231,7 @@ class Variant:
             out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(vn), vr(vt), sr(s_tail, 2)))
             out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(tmp), vr(V_OOB), sr(s_oob, 2)))
             src = vr(tmp)
-        pol = A_POLICY if is_a else B_POLICY
-        out.append("buffer_load_dwordx4 %s, %s, %s offen%s lds" % (src, sr(S_RA if is_a else S_RB, 4), sr(s_ka if is_a else s_kb),
-                                                                  (" " + pol) if pol else ""))
+        out.append("buffer_load_dwordx4 %s, %s, %s offen lds" % (src, sr(S_RA if is_a else S_RB, 4), sr(s_ka if is_a else s_kb)))
         return out
 
 
@@ -282,7 +247,8 @@ def m0_gaps(lines):
 
 def fixup(e, v, which, buf):
     """Zero the k elements outside the group's range in one 16-byte chunk per row (row = thread id) of
-    every operand that is contiguous along K.  which: 0 = first chunk of K tile 0, 1 = last chunk."""
+    every operand that is contiguous along K.  which: 0 = first chunk of K tile 0, 1 = last chunk.
+    buf: LDS buffer of the tile (ring: the addresses already point into the right slot, pass 0)."""
     for is_a in (True, False):
         tr = v.a_tr if is_a else v.b_tr
         if tr:
@@ -328,7 +294,7 @@ def interleave(e, mfmas, side_groups, need=None, prev_total=0):
         side = list(slots[k])
         if side and side[0].startswith("s_add_u32 m0"):
             lines.append(side.pop(0))
-        if need is not None and PARTIAL_WAITS:
+        if need is not None:
             allowed = prev_total - need[k] + issued
             if bound > allowed:
                 w = min(allowed, 15)
@@ -343,10 +309,8 @@ def interleave(e, mfmas, side_groups, need=None, prev_total=0):
         e(ins)
 
 
-def gen_variant(v):
-    use_regmap(v.waves)
-    e = Emit()
-    L = "%s_%%=" % v.name  # unique label suffix per asm instance
+def gen_classic_main(v, e, L):
+    """Prologue and K loop of the 128- and 64-row tiles: K tiles of 64 through three LDS buffers."""
     sT = S_T
     # temporaries
     s_kt, s_t1 = sT + 0, sT + 1
@@ -365,13 +329,8 @@ def gen_variant(v):
         e("s_cmp_ge_u32 %s, %s" % (sr(s_tile), sr(S_NK)))
         e("s_cselect_b64 %s, -1, 0" % sr(s_oob, 2))
 
-    def stamp(k):
-        if DBG_TIMING:
-            e("s_memrealtime %s" % sr(92 + 2 * k, 2))
-
     # ------------------------------------------------------------------ prologue
     e("; ---- prologue (%s)" % v.name)
-    stamp(0)
     e("v_mov_b32 %s, 0x80000000" % vr(V_OOB))
     # s[S_SPARE] = wave id | fix-up flags << 8 (bit 0: first chunk of the k range is partial, bit 1: last chunk)
     s_flags = sT + 18
@@ -415,7 +374,6 @@ def gen_variant(v):
         e("v_accvgpr_write_b32 a%d, 0" % r)
     e("s_waitcnt vmcnt(%d)" % ((S - 2) * v.ncopy + c3))
     e("s_barrier")
-    stamp(1)
     has_kc = not (v.a_tr and v.b_tr)
     if has_kc:
         # partial first / last chunk of a jagged k range (tile 0 is also the last tile when nk == 1)
@@ -444,9 +402,6 @@ def gen_variant(v):
 
     # ------------------------------------------------------------------ K loop, two tiles per trip
     need, nreads = v.read_need()
-    if DBG_NO_READS:
-        v.frag_reads = lambda *a: []
-        need, nreads = [0] * len(need), 0
 
     def ktile(buf, fast):
         # on entry: fragments of step 0 in set 0 (in flight); the first c3 copies of tile kt + S - 1 in flight.
@@ -468,35 +423,20 @@ def gen_variant(v):
         nb = (buf + 1) % S       # buffer of tile kt + 1
         cb = (buf + S - 1) % S   # buffer of tile kt + S - 1
         # step 0: MFMA set 0, read step 1 -> set 1, next copies of tile kt + S - 1
-        if not PARTIAL_WAITS:
-            e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 1, 1)]
         side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)]
         interleave(e, v.mfmas(0), side, need, nreads)
         # step 1
-        if not PARTIAL_WAITS:
-            e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 2, 0)]
         side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)]
         interleave(e, v.mfmas(1), side, need, nreads)
         # step 2
-        if not PARTIAL_WAITS:
-            e("s_waitcnt lgkmcnt(0)")
         side = [[x] for x in v.frag_reads(buf, 3, 1)]
         side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)]
-        npf = 0
-        if PREFETCH:
-            e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), PREFETCH))
-            e("s_mul_i32 %s, %s, %s" % (sr(sT + 16), sr(s_t1), sr(S_ASTEP)))
-            e("s_mul_i32 %s, %s, %s" % (sr(sT + 17), sr(s_t1), sr(S_BSTEP)))
-            side.append(["buffer_load_dword %s, %s, %s, %s offen" % (vr(V_PFD), vr(V_PF), sr(S_RA, 4), sr(sT + 16))])
-            side.append(["buffer_load_dword %s, %s, %s, %s offen" % (vr(V_PFD + 1), vr(V_PF + 1), sr(S_RB, 4), sr(sT + 17))])
-            npf = 2
         interleave(e, v.mfmas(0), side, need, nreads)
         # tile kt+1 has landed for this wave; after the barrier for all, and `buf` is free
-        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % (DBG_VMCNT if DBG_VMCNT >= 0 else (S - 2) * v.ncopy + npf))
-        if not DBG_NO_BARRIER:
-            e("s_barrier")
+        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % ((S - 2) * v.ncopy))
+        e("s_barrier")
         if not (v.a_tr and v.b_tr) and not fast:
             # the tile that has just landed is the last one and its last chunk is partial
             e("s_add_u32 %s, %s, 1" % (sr(s_t1), sr(s_kt)))
@@ -515,13 +455,12 @@ def gen_variant(v):
         e("s_add_u32 %s, %s, 1" % (sr(s_kt), sr(s_kt)))
 
     def ktile_both(buf):
-        if FAST_PATH:
-            e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), S))
-            e("s_cmp_lt_u32 %s, %s" % (sr(s_t1), sr(s_last)))
-            e("s_cbranch_scc0 L_slow%d_%s" % (buf, L))
-            ktile(buf, True)
-            e("s_branch L_join%d_%s" % (buf, L))
-            e.label("L_slow%d_%s" % (buf, L))
+        e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), S))
+        e("s_cmp_lt_u32 %s, %s" % (sr(s_t1), sr(s_last)))
+        e("s_cbranch_scc0 L_slow%d_%s" % (buf, L))
+        ktile(buf, True)
+        e("s_branch L_join%d_%s" % (buf, L))
+        e.label("L_slow%d_%s" % (buf, L))
         ktile(buf, False)
         e.label("L_join%d_%s" % (buf, L))
 
@@ -535,9 +474,165 @@ def gen_variant(v):
     e("s_cbranch_scc1 L_loop_%s" % L)
     e.label("L_done_%s" % L)
 
-    # ------------------------------------------------------------------ epilogue
+
+def merge_side(reads, copies):
+    """One list of side groups: the copy groups spread evenly among the fragment reads."""
+    total, nc = len(reads) + len(copies), len(copies)
+    at = {(j + 1) * total // nc - 1: j for j in range(nc)} if nc else {}
+    out, r = [], iter(reads)
+    for k in range(total):
+        out.append(copies[at[k]] if k in at else next(r))
+    return out
+
+
+def gen_ring_main(v, e, L):
+    """Prologue and K loop of the 256-row tile.  K is walked in half tiles of 32 (two k16 steps, 32 MFMAs
+    per wave) through a ring of four LDS slots per operand: while half h is multiplied, halves h + 1 and
+    h + 2 are in flight or landed and the copies of half h + 3 are issued, four per step, into the slot
+    that half h - 1 left at the last barrier.  Every copy therefore has two to three half tiles (2000 to
+    3000 cycles) to land, and the copies are spread evenly over the MFMAs instead of coming in bursts.
+    One barrier per half, after step 0: it publishes half h + 1 and releases the slot of half h."""
+    sT = S_T
+    s_h, s_t1 = sT + 0, sT + 1
+    s_ka, s_kb = sT + 2, sT + 3          # K offsets of the half whose copies are being issued
+    s_tail, s_oob = sT + 6, sT + 8       # pairs
+    s_last = sT + 14                     # nh - 1
+    s_zero = sT + 15
+    s_flags = sT + 18
+    s_waveA, s_waveB = sT + 20, sT + 21
+    NC = v.ncopy
+
+    def half_masks(s_half):
+        # tail mask: half == nh - 1 ; oob mask: half >= nh
+        e("s_cmp_eq_u32 %s, %s" % (sr(s_half), sr(s_last)))
+        e("s_cselect_b64 %s, -1, 0" % sr(s_tail, 2))
+        e("s_cmp_ge_u32 %s, %s" % (sr(s_half), sr(S_NK)))
+        e("s_cselect_b64 %s, -1, 0" % sr(s_oob, 2))
+
+    e("; ---- prologue (%s, ring)" % v.name)
+    e("v_mov_b32 %s, 0x80000000" % vr(V_OOB))
+    # s[S_SPARE] = wave id | flags << 8 (bit 0: first chunk of the k range is partial, bit 1: last chunk, bit 2: partial output chunks)
+    e("s_lshr_b32 %s, %s, 8" % (sr(s_flags), sr(S_SPARE)))
+    e("s_and_b32 %s, %s, 0xff" % (sr(sT + 19), sr(S_SPARE)))
+    e("s_sub_u32 %s, %s, 1" % (sr(s_last), sr(S_NK)))
+    e("s_mov_b32 %s, 0" % sr(s_zero))
+    e("s_mul_i32 %s, %s, %d" % (sr(s_waveA), sr(sT + 19), v.na * (TR_BLOCK if v.a_tr else 1024)))
+    e("s_add_u32 %s, %s, %s" % (sr(s_waveA), sr(s_waveA), sr(S_LDS)))
+    e("s_mul_i32 %s, %s, %d" % (sr(s_waveB), sr(sT + 19), v.nb * (TR_BLOCK if v.b_tr else 1024)))
+    e("s_add_u32 %s, %s, %s" % (sr(s_waveB), sr(s_waveB), sr(S_LDS)))
+    # halves 0, 1, 2 -> slots 0, 1, 2
+    for n in range(NC):
+        for ins in m0_gaps(v.dma(n, 0, "head", 0, 0, s_zero, s_zero, V_TMP)):
+            e(ins)
+    for hx in (1, 2):
+        e("s_mov_b32 %s, %d" % (sr(s_t1), hx))
+        half_masks(s_t1)
+        e("s_mul_i32 %s, %s, %d" % (sr(s_ka), sr(S_ASTEP), hx))
+        e("s_mul_i32 %s, %s, %d" % (sr(s_kb), sr(S_BSTEP), hx))
+        for n in range(NC):
+            for ins in m0_gaps(v.dma(n, hx, "loop", s_tail, s_oob, s_ka, s_kb, V_TMP + (n % 8))):
+                e(ins)
+    for r in range(16 * v.tm * v.tn):
+        e("v_accvgpr_write_b32 a%d, 0" % r)
+    e("s_waitcnt vmcnt(%d)" % (2 * NC))
+    e("s_barrier")
+    if not (v.a_tr and v.b_tr):
+        # partial first / last chunk of a jagged k range (half 0 is also the last half when nh == 1)
+        e("s_and_b32 %s, %s, 3" % (sr(s_t1), sr(s_flags)))
+        e("s_cmp_eq_u32 %s, 0" % sr(s_t1))
+        e("s_cbranch_scc1 L_nofix0_%s" % L)
+        e("s_bitcmp1_b32 %s, 0" % sr(s_flags))
+        e("s_cbranch_scc0 L_nohead_%s" % L)
+        fixup(e, v, 0, 0)
+        e("s_waitcnt lgkmcnt(0)")
+        e.label("L_nohead_%s" % L)
+        e("s_bitcmp1_b32 %s, 1" % sr(s_flags))
+        e("s_cbranch_scc0 L_notail0_%s" % L)
+        e("s_cmp_eq_u32 %s, 1" % sr(S_NK))
+        e("s_cbranch_scc0 L_notail0_%s" % L)
+        fixup(e, v, 1, 0)
+        e.label("L_notail0_%s" % L)
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_barrier")
+        e.label("L_nofix0_%s" % L)
+    for ins in v.frag_reads(0, 0, 0):
+        e(ins)
+    e("s_mov_b32 %s, 0" % sr(s_h))
+    e("s_cmp_eq_u32 %s, 0" % sr(S_NK))
+    e("s_cbranch_scc1 L_done_%s" % L)
+
+    need, nreads = v.read_need()
+
+    def half(slot, fast):
+        # on entry: fragments of step 0 in set 0 (in flight); halves h + 1, h + 2 in flight or landed
+        which = "fast" if fast else "loop"
+        e("; ---- half tile on slot %d%s" % (slot, " (interior)" if fast else ""))
+        e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_h), RING - 1))
+        if not fast:
+            half_masks(s_t1)
+        e("s_mul_i32 %s, %s, %s" % (sr(s_ka), sr(s_t1), sr(S_ASTEP)))
+        e("s_mul_i32 %s, %s, %s" % (sr(s_kb), sr(s_t1), sr(S_BSTEP)))
+        nxt = (slot + 1) % RING            # slot of half h + 1
+        dst = (slot + RING - 1) % RING     # slot of half h + 3 (= of half h - 1)
+        copies = [v.dma(n, dst, which, s_tail, s_oob, s_ka, s_kb, V_TMP + (n % 8)) for n in range(NC)]
+        # step 0: MFMA set 0, read step 1 -> set 1, first half of the copies
+        side = merge_side([[x] for x in v.frag_reads(slot, 1, 1)], copies[:NC // 2])
+        interleave(e, v.mfmas(0), side, need, nreads)
+        # half h + 1 has landed for this wave (the copies of halves h + 2 and h + 3 stay in flight); after
+        # the barrier it has for all waves, and everyone is done reading this slot
+        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % (NC + NC // 2))
+        e("s_barrier")
+        if not (v.a_tr and v.b_tr) and not fast:
+            # the half that has just landed is the last one and its last chunk is partial
+            e("s_add_u32 %s, %s, 1" % (sr(s_t1), sr(s_h)))
+            e("s_cmp_eq_u32 %s, %s" % (sr(s_t1), sr(s_last)))
+            e("s_cbranch_scc0 L_nofix%d_%s" % (slot + 1, L))
+            e("s_bitcmp1_b32 %s, 1" % sr(s_flags))
+            e("s_cbranch_scc0 L_nofix%d_%s" % (slot + 1, L))
+            fixup(e, v, 1, 0)
+            e("s_waitcnt lgkmcnt(0)")
+            e("s_barrier")
+            e.label("L_nofix%d_%s" % (slot + 1, L))
+        # step 1: MFMA set 1, read step 0 of the next half -> set 0, the other copies
+        side = merge_side([[x] for x in v.frag_reads(nxt, 0, 0)], copies[NC // 2:])
+        interleave(e, v.mfmas(1), side)
+        e("s_add_u32 %s, %s, 1" % (sr(s_h), sr(s_h)))
+
+    def half_both(slot):
+        e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_h), RING - 1))
+        e("s_cmp_lt_u32 %s, %s" % (sr(s_t1), sr(s_last)))
+        e("s_cbranch_scc0 L_slow%d_%s" % (slot, L))
+        half(slot, True)
+        e("s_branch L_join%d_%s" % (slot, L))
+        e.label("L_slow%d_%s" % (slot, L))
+        half(slot, False)
+        e.label("L_join%d_%s" % (slot, L))
+
+    e.label("L_loop_%s" % L)
+    for slot in range(RING - 1):
+        half_both(slot)
+        e("s_cmp_ge_u32 %s, %s" % (sr(s_h), sr(S_NK)))
+        e("s_cbranch_scc1 L_done_%s" % L)
+    half_both(RING - 1)
+    e("s_cmp_lt_u32 %s, %s" % (sr(s_h), sr(S_NK)))
+    e("s_cbranch_scc1 L_loop_%s" % L)
+    e.label("L_done_%s" % L)
+
+
+def gen_variant(v):
+    e = Emit()
+    L = "%s_%%=" % v.name  # unique label suffix per asm instance
+    if v.ring:
+        gen_ring_main(v, e, L)
+    else:
+        gen_classic_main(v, e, L)
+    gen_epilogue(v, e, L)
+    return e
+
+
+def gen_epilogue(v, e, L):
     e("; ---- epilogue")
-    stamp(2)
+    t = V_TMP
     e("s_waitcnt vmcnt(0) lgkmcnt(0)")
     e("s_nop 15")
     e("s_nop 15")
@@ -549,15 +644,15 @@ def gen_variant(v):
         # v[V_EPI + 2] = store offset of the lane's row in read-back instruction 0 (or OOB when the lane's
         #                columns are invalid); v[V_EPI + 3] = that row - row_lo, valid iff (unsigned) < S_ROWCNT
         t = V_TMP
-        pitch = PITCH if v.waves == 4 else PITCH8
-        ipp = v.tm if v.waves == 4 else 2
+        pitch = PITCH
+        ipp = v.tm
         rpi = 16 // v.tn          # rows per read-back instruction (64 lanes x 16 bytes over rows of 32 tn columns)
         depth = 4
         regs = [t + 4 * x for x in range(depth)]          # read-back data, 4 registers each
         voff, vrow, vsel = t + 24, t + 25, t + 26
         e("v_mov_b32 %s, %s" % (vr(voff), vr(V_EPI + 2)))
         e("v_mov_b32 %s, %s" % (vr(vrow), vr(V_EPI + 3)))
-        partial = v.waves == 4
+        partial = True
         if partial:
             # A group boundary that is not a multiple of 8 columns leaves 16-byte chunks of which only some
             # elements belong to this tile (flag bit 2 of the tile): those go out as 2-byte stores.
@@ -644,10 +739,8 @@ def gen_variant(v):
                         e("s_and_b64 vcc, %s, %s" % (sr(S_T + 32, 2), sr(S_T + 24 + 2 * j, 2)))
                         e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(t + 8 + (k % 8)), vr(V_OOB), vr(V_EPI + 2)))
                         e("buffer_store_dword %s, %s, %s, %s offen offset:%d" % (vr(b), vr(t + 8 + (k % 8)), sr(S_RC, 4), sr(S_T + 16), 128 * j))
-    stamp(3)
     e("s_waitcnt lgkmcnt(0)")
     e("s_barrier")
-    return e
 
 
 def clobbers(v):
@@ -668,31 +761,22 @@ def main():
     out.append("#define GMM_TILE_TR_STAGE %d" % TR_STAGE)
     out.append("#define GMM_TILE_STAGING_BYTES %d" % STAGE_BYTES)
     out.append("#define GMM_TILE_STAGES_SHORT %d" % STAGES_SHORT)
-    out.append("#define GMM_TILE_PITCH8 %d" % PITCH8)
-    for a_tr, b_tr, f32, tm, waves, f16 in [(a, b, f, t, w, h) for h in (0, 1) for w in (4, 8) for a in (0, 1) for b in (0, 1)
-                                            for f in (0, 1) for t in (4, 2, 1)]:
-        if (tm != 4 and (a_tr or waves == 8)) or (f16 and waves == 8):
-            continue
-        v = Variant(a_tr, b_tr, f32, tm, waves, f16)
-        e = gen_variant(v)
-        out.append("")
-        if waves == 4:
+    for f16 in (0, 1):
+        for a_tr, b_tr, f32, tm in [(a, b, f, t) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1)]:
+            if tm != 4 and a_tr:
+                continue
+            v = Variant(a_tr, b_tr, f32, tm, f16)
+            e = gen_variant(v)
+            out.append("")
             out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm, f16))
-        else:
-            out.append("template <> __device__ __forceinline__ void gmm_tile_asm8<%d, %d, %d>(GmmTileRegs8& r) {" % (a_tr, b_tr, f32))
-        out.append("  asm volatile(")
-        out.append(e.text())
-        out.append('      : "={s[92:99]}"(r.stamps)' if DBG_TIMING else "      :")
-        if waves == 4:
+            out.append("  asm volatile(")
+            out.append(e.text())
+            out.append("      :")
             out.append('      : "{v[128:135]}"(r.voa_head), "{v[136:143]}"(r.vob_head), "{v[144:151]}"(r.voa), "{v[152:159]}"(r.vob),')
             out.append('        "{v[160:167]}"(r.voa_tail), "{v[168:175]}"(r.vob_tail), "{v[176:179]}"(r.ra_addr), "{v[180:183]}"(r.rb_addr),')
-            out.append('        "{v[184:187]}"(r.epi), "{v[190:191]}"(r.epi2), "{v[192:193]}"(r.pf), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
-        else:
-            out.append('      : "{v[80:83]}"(r.voa_head), "{v[84:87]}"(r.vob_head), "{v[88:91]}"(r.voa), "{v[92:95]}"(r.vob),')
-            out.append('        "{v[96:99]}"(r.voa_tail), "{v[100:103]}"(r.vob_tail), "{v[104:107]}"(r.ra_addr), "{v[108:111]}"(r.rb_addr),')
-            out.append('        "{v[112:115]}"(r.epi), "{v[116:119]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
-        out.append("      : %s);" % clobbers(v))
-        out.append("}")
+            out.append('        "{v[184:187]}"(r.epi), "{v[190:191]}"(r.epi2), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
+            out.append("      : %s);" % clobbers(v))
+            out.append("}")
     sys.stdout.write("\n".join(out) + "\n")
 
 

@@ -84,13 +84,14 @@ bool asm_tile_eligible(const Problem& pr, const GmmLayout& lay) {
 
 int run(Problem& pr, hipStream_t stream) {
   GmmParams& p = pr.p;
-  if (!p.a || !p.b || !p.c) return GMM_ERR_BAD_ARGUMENT;
-  if (p.jag != GMM_JAG_NONE && (!p.offs || p.G < 1 || p.G >= GMM_MAX_GROUPS)) return GMM_ERR_BAD_ARGUMENT;
-  if (p.G < 0) return GMM_ERR_BAD_ARGUMENT;
+  if (p.G < 0 || (p.G >= GMM_MAX_GROUPS && p.jag != GMM_JAG_NONE)) return GMM_ERR_BAD_ARGUMENT;
   if (pr.in_dtype < 0 || pr.in_dtype > GMM_DT_F32) return GMM_ERR_UNSUPPORTED;
   if (pr.out_dtype != pr.in_dtype && pr.out_dtype != GMM_DT_F32) return GMM_ERR_UNSUPPORTED;
-  // Nothing to write.
+  // Nothing to write: no groups (the reference launches and stores nothing, kernels.py:162-172 with
+  // G == 0 finds no owner for any row), or an empty extent.  Empty tensors may come with null pointers.
   if (p.G == 0 || p.M == 0 || p.N == 0) return GMM_OK;
+  if (!p.a || !p.b || !p.c) return GMM_ERR_BAD_ARGUMENT;
+  if (p.jag != GMM_JAG_NONE && !p.offs) return GMM_ERR_BAD_ARGUMENT;
 
   const int cus = device_cus();
   if (cus <= 0) return GMM_ERR_LAUNCH;
@@ -100,7 +101,7 @@ int run(Problem& pr, hipStream_t stream) {
   const int forced = g_forced_path.load(std::memory_order_relaxed);
   const bool aligned = mfma_eligible(pr, lay, align);
   const bool can_asm = aligned && asm_tile_eligible(pr, lay);
-  // fp16 has the assembly tile only (configuration 1); bf16 also the register-staged kernel and the 8-wave tile
+  // fp16 has the assembly tile only (configuration 1); bf16 also the register-staged kernel
   const bool can_mfma = aligned && (pr.in_dtype == GMM_DT_BF16 || can_asm);
   if (forced == GMM_PATH_MFMA && !can_mfma) return GMM_ERR_UNSUPPORTED;
   const bool use_mfma = can_mfma && forced != GMM_PATH_GENERIC;
@@ -110,11 +111,9 @@ int run(Problem& pr, hipStream_t stream) {
     p.align = align;
     p.xcd_remap = g_xcd_remap.load(std::memory_order_relaxed);
     int cfg = g_forced_config.load(std::memory_order_relaxed);
-    if ((cfg == GMM_CFG_ASM_256x256 || cfg == GMM_CFG_ASM8_256x256) && !can_asm) return GMM_ERR_UNSUPPORTED;
+    if (cfg == GMM_CFG_ASM_256x256 && !can_asm) return GMM_ERR_UNSUPPORTED;
     if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = can_asm ? GMM_CFG_ASM_256x256 : GMM_CFG_REG_256x256;
     if (pr.in_dtype != GMM_DT_BF16 && cfg != GMM_CFG_ASM_256x256) return GMM_ERR_UNSUPPORTED;
-    // the 8-wave tile has no element-masked stores for group boundaries inside a 16-byte chunk
-    if (cfg == GMM_CFG_ASM8_256x256 && p.jag == GMM_JAG_N) return GMM_ERR_UNSUPPORTED;
     // the assembly tile stores 16-byte chunks: its tile columns start at multiples of 8 elements
     if (cfg == GMM_CFG_ASM_256x256 && p.jag == GMM_JAG_N) p.align = 8;
     // Tile heights of the assembly tile: 256-row tiles unless the launch would not even fill four rounds
@@ -222,9 +221,8 @@ int gmm_set_mfma_config(int config) { return g_forced_config.exchange(config); }
 int gmm_last_mfma_config(void) { return t_last_config; }
 int gmm_set_xcd_remap(int on) { return g_xcd_remap.exchange(on ? 1 : 0); }
 int gmm_set_tile_heights(int tall, int shrt) {
-  g_forced_tall.store(tall);
-  g_forced_short.store(shrt);
-  return 0;
+  const int prev_tall = g_forced_tall.exchange(tall), prev_short = g_forced_short.exchange(shrt);
+  return ((prev_tall + 1) << 16) | ((prev_short + 1) & 0xffff);
 }
 
 int64_t gmm_host_tile_list(const int32_t* offs_host, int32_t G, int32_t jagged, int32_t M, int32_t N, int32_t K,

@@ -70,26 +70,6 @@ __device__ __forceinline__ GmmTile gmm_locate_tile(const GmmParams& p, const int
   return gmm_make_tile(p, g, lo, hi, mt, nt, bm, bn);
 }
 
-// Same, for a tile id that differs from lane to lane (no cross-lane broadcasts).
-__device__ __forceinline__ GmmTile gmm_locate_tile_divergent(const GmmParams& p, const int32_t* cum, int t, int bm, int bn) {
-  int g, local, lo = 0, hi = 0, tm, tn;
-  if (p.jag == GMM_JAG_NONE) {
-    tm = gmm_cdiv(p.M, bm);
-    tn = gmm_cdiv(p.N, bn);
-    g = t / (tm * tn);
-    local = t - g * (tm * tn);
-  } else {
-    const int extent = p.jag == GMM_JAG_M ? p.M : (p.jag == GMM_JAG_N ? p.N : p.K);
-    g = gmm_find_group(cum, p.G, t);
-    local = t - cum[g];
-    gmm_group_range(p.offs, g, extent, lo, hi);
-    gmm_group_grid(p.jag, lo, hi, p.M, p.N, bm, bn, p.align, tm, tn);
-  }
-  int mt, nt;
-  gmm_decode_in_group(local, tm, tn, mt, nt);
-  return gmm_make_tile(p, g, lo, hi, mt, nt, bm, bn);
-}
-
 // ---- two-height tile list (gmm_sched.h): tables cum[0] (tall) and cum[1] (short), each G + 1 entries ---- //
 template <int NT>
 __device__ __forceinline__ void gmm_scan_table(int32_t* cum) {

@@ -17,9 +17,7 @@ struct GmmLayout {
 // REG: tiles staged through registers, compiler-scheduled (takes every aligned layout and the
 //      jagged-column / unaligned jagged-contraction cases).
 // ASM: generated assembly tile with direct-to-LDS copies (the fast one).
-enum GmmMfmaConfig : int { GMM_CFG_REG_256x256 = 0, GMM_CFG_ASM_256x256 = 1, GMM_CFG_ASM8_256x256 = 2, GMM_CFG_COUNT };
+enum GmmMfmaConfig : int { GMM_CFG_REG_256x256 = 0, GMM_CFG_ASM_256x256 = 1, GMM_CFG_COUNT };
 
 // bf16 inputs only; out_dtype bf16 or fp32.  Returns like gmm_launch_generic.
 int gmm_launch_mfma(GmmParams p, GmmLayout lay, int in_dtype, int out_dtype, int config, int num_cus, hipStream_t stream);
-// Tile edge (rows, columns) of a configuration.
-void gmm_mfma_tile_shape(int config, int& bm, int& bn);

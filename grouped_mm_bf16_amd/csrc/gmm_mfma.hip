@@ -261,13 +261,13 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) gmm_mfma_kernel(cons
 // Same tile list, but each tile's main loop and epilogue run as one hand-scheduled assembly block:
 // direct global -> LDS copies, no register staging, explicit registers.  A_TR / B_TR: the operand is
 // contiguous along M / N (not along K) and is read from LDS with transposing loads.
-// TALL_TM: height of the tall tiles in units of 64 rows (4 or 2); 64-row short tiles for group remainders
-// exist when A is contiguous along K (p.shrt == 64).
-// WAVES = 4: one wave per SIMD, tiles of 256, 128 and 64 rows share the launch (a column-major A has only
-// the first).  WAVES = 8: two waves per SIMD, 256-row tiles only (the launcher sets p.shrt = 0).
-template <int A_TR, int B_TR, int OUT_F32, int WAVES, int F16>
-__global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams p) {
-  constexpr bool SHORT_TILES = !A_TR && WAVES == 4;
+// One wave per SIMD; tiles of 256, 128 and 64 rows share the launch when A is contiguous along K (a
+// column-major A has only the first): p.tall is the height of the tall tiles (256 or 128), p.shrt == 64
+// turns on the 64-row tiles for group remainders.
+template <int A_TR, int B_TR, int OUT_F32, int F16>
+__global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
+  constexpr int WAVES = 4;
+  constexpr bool SHORT_TILES = !A_TR;
   constexpr int LDS_256 = gmm_tile_lds_bytes<A_TR, B_TR, 4>();
   constexpr int LDS_128 = SHORT_TILES ? gmm_tile_lds_bytes<0, B_TR, 2>() : 0;
   constexpr int LDS_64 = SHORT_TILES ? gmm_tile_lds_bytes<0, B_TR, 1>() : 0;
@@ -328,23 +328,25 @@ __global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams 
       GmmTileDesc dsc;
       dsc.a.ld = lda;
       dsc.b.ld = ldb;
+      // Extents end at the last element of the operand's last row, not at a whole leading dimension: a
+      // padded view (ld larger than the row) may end exactly there.
       if (!A_TR) {
         dsc.a.base = a + int64_t(m0) * lda + k_begin;
-        dsc.a.bytes = (int64_t(p.M - m0) * lda - k_begin) * 2;
+        dsc.a.bytes = (int64_t(p.M - 1 - m0) * lda + (p.K - k_begin)) * 2;
       } else {
         dsc.a.base = a + int64_t(k_begin) * lda + m0;
-        dsc.a.bytes = (int64_t(p.K - k_begin) * lda - m0) * 2;
+        dsc.a.bytes = (int64_t(p.K - 1 - k_begin) * lda + (p.M - m0)) * 2;
       }
       if (!B_TR) {
         dsc.b.base = b + int64_t(n0) * ldb + k_begin;
-        dsc.b.bytes = (int64_t(p.N - n0) * ldb - k_begin) * 2;
+        dsc.b.bytes = (int64_t(p.N - 1 - n0) * ldb + (p.K - k_begin)) * 2;
       } else {
         dsc.b.base = b + int64_t(k_begin) * ldb + n0;
-        dsc.b.bytes = (int64_t(p.K - k_begin) * ldb - n0) * 2;
+        dsc.b.bytes = (int64_t(p.K - 1 - k_begin) * ldb + (p.N - n0)) * 2;
       }
       dsc.c = C + (int64_t(g) * p.c_sg + int64_t(m0) * ldc + n0) * ESZ;
       dsc.ldc = ldc;
-      dsc.c_bytes = (int64_t(p.M - m0) * ldc - n0) * ESZ;
+      dsc.c_bytes = (int64_t(p.M - 1 - m0) * ldc + (p.N - n0)) * ESZ;
       dsc.klen = k_hi > k_lo ? k_hi - k_begin : 0;
       dsc.khead = k_lo - k_begin;
       dsc.row_rel0 = m0 - m_lo;
@@ -352,9 +354,7 @@ __global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams 
       dsc.row_cnt = gmm_min(m_hi, m0 + rows) - m_lo;
       dsc.col_lo = gmm_max(n_lo - n0, 0);
       dsc.col_hi = gmm_min(n_hi - n0, GMM_TILE_N);
-      if constexpr (WAVES == 8) {
-        gmm_tile_compute8<A_TR, B_TR, OUT_F32>(dsc, lds_base, lane_j, wave);
-      } else if constexpr (A_TR) {
+      if constexpr (A_TR) {
         gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16>(dsc, lds_base, lane_j, wave);
       } else {
         if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16>(dsc, lds_base, lane_j, wave);
@@ -367,17 +367,17 @@ __global__ void __launch_bounds__(WAVES * 64, 1) gmm_asm_kernel(const GmmParams 
   }
 }
 
-template <int OUT_F32, int WAVES, int F16>
+template <int OUT_F32, int F16>
 int launch_asm(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
-  const dim3 grid(p.num_wg), block(WAVES * 64);
+  const dim3 grid(p.num_wg), block(256);
   if (lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32, WAVES, F16>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32, F16>), grid, block, 0, stream, p);
   else if (lay.a_kc && !lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32, WAVES, F16>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<0, 1, OUT_F32, F16>), grid, block, 0, stream, p);
   else if (!lay.a_kc && lay.b_kc)
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32, WAVES, F16>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 0, OUT_F32, F16>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32, WAVES, F16>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gmm_asm_kernel<1, 1, OUT_F32, F16>), grid, block, 0, stream, p);
   return hipGetLastError() == hipSuccess ? 0 : 1;
 }
 
@@ -398,12 +398,6 @@ int launch_layout(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
 
 }  // namespace
 
-void gmm_mfma_tile_shape(int config, int& bm, int& bn) {
-  (void)config;
-  bm = 256;
-  bn = 256;
-}
-
 int gmm_launch_mfma(GmmParams p, GmmLayout lay, int in_dtype, int out_dtype, int config, int num_cus, hipStream_t stream) {
   // persistent grid: one workgroup per CU, fewer (a multiple of 8, for the XCD renumbering) when the launch
   // cannot have that many tiles
@@ -418,16 +412,11 @@ int gmm_launch_mfma(GmmParams p, GmmLayout lay, int in_dtype, int out_dtype, int
     // a column-major A has only the 256-row tile
     if (!lay.a_kc) { p.tall = 256; p.shrt = 0; }
     if (p.tall != 128) p.tall = 256;
-    if (in_dtype == GMM_DT_BF16) return out16 ? launch_asm<0, 4, 0>(p, lay, stream) : launch_asm<1, 4, 0>(p, lay, stream);
-    if (in_dtype == GMM_DT_F16) return out16 ? launch_asm<0, 4, 1>(p, lay, stream) : launch_asm<1, 4, 1>(p, lay, stream);
+    if (in_dtype == GMM_DT_BF16) return out16 ? launch_asm<0, 0>(p, lay, stream) : launch_asm<1, 0>(p, lay, stream);
+    if (in_dtype == GMM_DT_F16) return out16 ? launch_asm<0, 1>(p, lay, stream) : launch_asm<1, 1>(p, lay, stream);
     return -1;
   }
-  if (in_dtype != GMM_DT_BF16) return -1;     // the other configurations are bf16 only
-  if (config == GMM_CFG_ASM8_256x256) {
-    p.tall = 256;
-    p.shrt = 0;
-    return out16 ? launch_asm<0, 8, 0>(p, lay, stream) : launch_asm<1, 8, 0>(p, lay, stream);
-  }
+  if (in_dtype != GMM_DT_BF16) return -1;     // the register-staged kernel is bf16 only
   if (out16) return launch_layout<256, 256, 2, 2, uint16_t>(p, lay, stream);
   return launch_layout<256, 256, 2, 2, float>(p, lay, stream);
 }

@@ -17,32 +17,16 @@ struct GmmTileRegs {
   gmm_v4i epi;                 // epilogue: per-lane addresses (see gen_tile_asm.py)
   gmm_v2i epi2;                // bf16 epilogue: store offset of the lane's chunk whatever its validity; mask of
                                // its valid elements when only some of them are (a group boundary inside it)
-  gmm_v2i pf;                  // L2 prefetch offsets of this lane for A and B
   gmm_v4i fix;                 // LDS addresses of this thread's row in the first / last k chunk (A, A, B, B)
   gmm_v8i masks;               // keep-masks of the first and of the last 16-byte k chunk
   gmm_v4i rsrc_a, rsrc_b, rsrc_c;
   gmm_v8i scal;                // nk, a_step, b_step, lds_base, row_cnt, c_step, n_valid, wave
-  gmm_v8i stamps;              // timing builds only: four 64-bit s_memrealtime stamps
 };
 
 // TM = MFMA block rows per wave: the tile is 64 * TM rows (256, 128 or 64) by 256 columns.
 // F16 = 1: A, B and a 16-bit output are fp16 instead of bf16 (same layouts, other MFMA and conversion).
 template <int A_TR, int B_TR, int OUT_F32, int TM, int F16>
 __device__ __forceinline__ void gmm_tile_asm(GmmTileRegs& r);
-
-// Same for the 8-wave form of the 256 x 256 tile (two waves per SIMD, 128 x 64 per wave): every wave
-// issues half as many copies, so the offset vectors are 4 wide.
-struct GmmTileRegs8 {
-  gmm_v4i voa_head, vob_head, voa, vob, voa_tail, vob_tail;
-  gmm_v4i ra_addr, rb_addr, epi, fix;
-  gmm_v8i masks;
-  gmm_v4i rsrc_a, rsrc_b, rsrc_c;
-  gmm_v8i scal;
-  gmm_v8i stamps;
-};
-
-template <int A_TR, int B_TR, int OUT_F32>
-__device__ __forceinline__ void gmm_tile_asm8(GmmTileRegs8& r);
 
 #include "gmm_tile_asm.inc"
 
@@ -144,8 +128,7 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int
 }
 
 template <int A_TR, int B_TR, int OUT_F32, int TM = 4, int F16 = 0>
-__device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave,
-                                                 gmm_v8i* stamps = nullptr) {
+__device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave) {
   static_assert(TM == 4 || !A_TR, "short tiles exist for a K-contiguous A only");
   constexpr int WROWS = 32 * TM;  // rows of the tile per wave row
   constexpr int B_BASE = GmmTileLayout<A_TR, TM>::b_base;
@@ -171,9 +154,6 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
       r.rb_addr[s] = lds_base + B_BASE + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wn * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
     }
   }
-  // L2 prefetch: 256 cache lines per operand and K tile, one per lane
-  r.pf[0] = A_TR ? (wave * 16 + (lane >> 2)) * t.a.ld * 2 + (lane & 3) * 128 : (wave * 64 + lane) * t.a.ld * 2;
-  r.pf[1] = B_TR ? (wave * 16 + (lane >> 2)) * t.b.ld * 2 + (lane & 3) * 128 : (wave * 64 + lane) * t.b.ld * 2;
   int c_step, n_valid = 0, partial = 0;
   r.epi2[0] = 0;
   r.epi2[1] = 0;
@@ -235,106 +215,4 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
 #pragma unroll
   for (int i = 0; i < 8; ++i) r.scal[i] = __builtin_amdgcn_readfirstlane(sc[i]);
   gmm_tile_asm<A_TR, B_TR, OUT_F32, TM, F16>(r);
-  if (stamps) *stamps = r.stamps;
-}
-
-// ---- 8 waves: wave = wm + 2 wn, wm in 0..1 (128 rows), wn in 0..3 (64 columns) -------------------------- //
-template <int TR>
-__device__ __forceinline__ void gmm_copy_offsets8(int lane, int wave, int ld, int klen, int khead, int nk,
-                                                  gmm_v4i& head, gmm_v4i& full, gmm_v4i& tail) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int k, vo;
-    if (!TR) {
-      const int row = wave * 32 + i * 8 + (lane >> 3);
-      const int c = (lane & 7) ^ gmm_swz(row);
-      k = c * 8;
-      vo = row * ld * 2 + c * 16;
-    } else {
-      const int blk = wave * 4 + i;
-      k = 8 * (blk >> 2) + (blk & 3) + 4 * (lane >> 5);
-      vo = k * ld * 2 + (lane & 31) * 16;
-    }
-    const bool before = TR && k < khead;
-    full[i] = vo;
-    head[i] = (k < klen && !before) ? vo : (int)GMM_OOB;
-    tail[i] = ((nk - 1) * GMM_TILE_K + k < klen && !(before && nk == 1)) ? vo : (int)GMM_OOB;
-  }
-}
-
-template <int A_TR, int B_TR, int OUT_F32>
-__device__ __forceinline__ void gmm_tile_compute8(const GmmTileDesc& t, unsigned lds_base, int lane, int wave,
-                                                  gmm_v8i* stamps = nullptr) {
-  constexpr int B_BASE = GmmTileLayout<A_TR, 4>::b_base;
-  const int wm = wave & 1, wn = wave >> 1;
-  const int nk = (t.klen + GMM_TILE_K - 1) / GMM_TILE_K;
-  GmmTileRegs8 r;
-  gmm_copy_offsets8<A_TR>(lane, wave, t.a.ld, t.klen, t.khead, nk, r.voa_head, r.voa, r.voa_tail);
-  gmm_copy_offsets8<B_TR>(lane, wave, t.b.ld, t.klen, t.khead, nk, r.vob_head, r.vob, r.vob_tail);
-  const int q = lane >> 4, ii = lane & 15;
-#pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const int chunk = 2 * s + (lane >> 5);
-    if (!A_TR) {
-      const int row = wm * 128 + (lane & 31);
-      r.ra_addr[s] = lds_base + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
-    } else {
-      r.ra_addr[s] = lds_base + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wm * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
-    }
-    if (!B_TR) {
-      const int row = wn * 64 + (lane & 31);
-      r.rb_addr[s] = lds_base + B_BASE + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
-    } else {
-      r.rb_addr[s] = lds_base + B_BASE + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wn * 64 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
-    }
-  }
-  int c_step, n_valid = 0;
-  if (!OUT_F32) {
-    // staging: 64 rows of 64 columns per wave and pass; read back 8 rows per instruction
-    const int row_t = wm * 128 + (lane >> 3), col_t = wn * 64 + (lane & 7) * 8;
-    const unsigned stage = lds_base + wave * (64 * GMM_TILE_PITCH8);
-    r.epi[0] = stage + (lane & 31) * GMM_TILE_PITCH8 + 8 * (lane >> 5);
-    r.epi[1] = stage + (lane >> 3) * GMM_TILE_PITCH8 + (lane & 7) * 16;
-    r.epi[2] = (col_t >= t.col_lo && col_t + 8 <= t.col_hi) ? (row_t * t.ldc + col_t) * 2 : (int)GMM_OOB;
-    r.epi[3] = t.row_rel0 + row_t;
-    c_step = 8 * t.ldc * 2;
-  } else {
-    const int row_t = wm * 128 + 4 * (lane >> 5), col_t = wn * 64 + (lane & 31);
-    r.epi[0] = 0;
-    r.epi[1] = lane & 31;
-    r.epi[2] = (row_t * t.ldc + col_t) * 4;
-    r.epi[3] = t.row_rel0 + row_t;
-    c_step = t.ldc * 4;
-    n_valid = t.col_hi - wn * 64;
-    if (n_valid < 0) n_valid = 0;
-  }
-  r.rsrc_a = gmm_make_rsrc(t.a.base, t.a.bytes);
-  r.rsrc_b = gmm_make_rsrc(t.b.base, t.b.bytes);
-  r.rsrc_c = gmm_make_rsrc(t.c, t.c_bytes);
-  const int a_step = A_TR ? GMM_TILE_K * t.a.ld * 2 : GMM_TILE_K * 2;
-  const int b_step = B_TR ? GMM_TILE_K * t.b.ld * 2 : GMM_TILE_K * 2;
-  const int ktail = t.klen & 7;
-  int flags = 0;
-  if (!(A_TR && B_TR)) flags = (t.khead ? 1 : 0) | (ktail ? 2 : 0);
-  {
-    // one row of each operand tile per thread pair (both write the same masked value)
-    const int row = (wave * 64 + lane) & 255;
-    const int c_last = ((t.klen - 1) & (GMM_TILE_K - 1)) >> 3;
-    r.fix[0] = lds_base + row * 128 + ((0 ^ gmm_swz(row)) << 4);
-    r.fix[1] = lds_base + row * 128 + ((c_last ^ gmm_swz(row)) << 4);
-    r.fix[2] = lds_base + B_BASE + row * 128 + ((0 ^ gmm_swz(row)) << 4);
-    r.fix[3] = lds_base + B_BASE + row * 128 + ((c_last ^ gmm_swz(row)) << 4);
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const unsigned h0 = (2 * w >= t.khead) ? 0x0000ffffu : 0u, h1 = (2 * w + 1 >= t.khead) ? 0xffff0000u : 0u;
-      const unsigned t0 = (2 * w < ktail) ? 0x0000ffffu : 0u, t1 = (2 * w + 1 < ktail) ? 0xffff0000u : 0u;
-      r.masks[w] = __builtin_amdgcn_readfirstlane((int)(h0 | h1));
-      r.masks[4 + w] = __builtin_amdgcn_readfirstlane((int)(t0 | t1));
-    }
-  }
-  const int sc[8] = {nk, a_step, b_step, (int)lds_base, t.row_cnt, c_step, n_valid, wave | (flags << 8)};
-#pragma unroll
-  for (int i = 0; i < 8; ++i) r.scal[i] = __builtin_amdgcn_readfirstlane(sc[i]);
-  gmm_tile_asm8<A_TR, B_TR, OUT_F32>(r);
-  if (stamps) *stamps = r.stamps;
 }

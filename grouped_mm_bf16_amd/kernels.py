@@ -74,6 +74,12 @@ def _launch_now(variant: int, a: torch.Tensor, b: torch.Tensor, offs: Optional[t
 _launch_op = torch.library.custom_op("grouped_mm_bf16_amd::launch", mutates_args=("out",))(_launch_now)
 
 
+@_launch_op.register_fake
+def _launch_fake(variant, a, b, offs, out) -> None:
+    """Shape propagation under FakeTensor: the op returns nothing and only fills `out`."""
+    return None
+
+
 def _launch(variant: int, a: torch.Tensor, b: torch.Tensor, offs: Optional[torch.Tensor], out: torch.Tensor) -> None:
     if torch.compiler.is_compiling():
         _launch_op(variant, a, b, offs, out)
@@ -141,11 +147,11 @@ def forced_mfma_config(config: int):
 def forced_tile_heights(tall: int, shrt: int):
     """Force the tile heights of the assembly tile (tall 256 / 128, short 64 / 0; -1 = automatic)."""
     lib = _lib.load()
-    lib.gmm_set_tile_heights(tall, shrt)
+    prev = lib.gmm_set_tile_heights(tall, shrt)   # ((tall + 1) << 16) | (short + 1) of the previous setting
     try:
         yield
     finally:
-        lib.gmm_set_tile_heights(-1, -1)
+        lib.gmm_set_tile_heights((prev >> 16) - 1, (prev & 0xffff) - 1)
 
 
 def last_path() -> str:

@@ -17,7 +17,7 @@
  *   - `stream` is a hipStream_t (NULL = the default stream);
  *   - the return value is a gmm_status; nothing is thrown across the boundary.
  *   - elements that no group owns (rows / columns at or beyond offs[G-1]) are
- *     not written.
+ *     not written; with G == 0 nothing is written and GMM_OK is returned.
  */
 #ifndef GROUPED_MM_HIP_H
 #define GROUPED_MM_HIP_H
@@ -95,13 +95,14 @@ int gmm_3d2d(const void* a, const void* b, void* out, const int32_t* offs, int32
 int gmm_set_path(int path);
 int gmm_last_path(void);
 /* Tile configuration of the MFMA family: -1 = choose from the shapes, 0 = register-staged kernel,
- * 1 = assembly tile with 4 waves (256 / 128 / 64-row tiles), 2 = assembly tile with 8 waves (256-row tiles). */
+ * 1 = assembly tile (256 / 128 / 64-row tiles).  Returns the previous setting. */
 int gmm_set_mfma_config(int config);
 int gmm_last_mfma_config(void);
 /* 0 / 1: renumber tiles per XCD (default 1). */
 int gmm_set_xcd_remap(int on);
 /* Tile heights of the assembly tile: tall = 256 or 128 (-1: chosen from the shapes), shrt = 64 or 0
- * (-1: 64 whenever the first operand is contiguous along the contraction). */
+ * (-1: 64 whenever the first operand is contiguous along the contraction).  Returns the previous
+ * setting packed as ((tall + 1) << 16) | (shrt + 1). */
 int gmm_set_tile_heights(int tall, int shrt);
 
 /* Host-side run of the tile scheduler that the kernels execute on the device:

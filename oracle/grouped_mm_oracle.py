@@ -144,8 +144,8 @@ RTOL = 1.6e-2
 
 
 def atol_for_k(k: int) -> float:
-    """atol = 1e-2 * sqrt(K / 64), K = contraction length (at least 64)."""
-    return 1e-2 * math.sqrt(max(int(k), 64) / 64.0)
+    """atol = 1e-2 * sqrt(K / 64), K = contraction length of the compared elements."""
+    return 1e-2 * math.sqrt(max(int(k), 0) / 64.0)
 
 
 def assert_close(actual: torch.Tensor, expected: torch.Tensor, k: int, what: str = "") -> None:
@@ -156,3 +156,13 @@ def assert_close(actual: torch.Tensor, expected: torch.Tensor, k: int, what: str
     owned = ~torch.isnan(expected)
     torch.testing.assert_close(actual[owned], expected[owned], rtol=RTOL, atol=atol_for_k(k),
                                msg=lambda m: f"{what}: {m}")
+
+
+def assert_close_grouped(actual: torch.Tensor, expected: torch.Tensor, a, b, offs, what: str = "") -> None:
+    """`assert_close` with K taken per element: the contraction length of the element's own group.
+    Only the K-grouped variant (2-D x 2-D) has groups with different K; the others use the shared K."""
+    if a.dim() == 2 and b.dim() == 2:
+        for g, (s, e) in enumerate(group_ranges(offs.tolist())):
+            assert_close(actual[g], expected[g], e - s, what=f"{what} group {g} (K={e - s})")
+    else:
+        assert_close(actual, expected, a.shape[-1], what=what)

@@ -41,12 +41,16 @@ def run_poisoned(variant_fn, a, b, offs, shape, dtype):
     return out.cpu()
 
 
-def check(out, a, b, offs, k, path=None):
+def check(out, a, b, offs, k=None, path=None, what=""):
+    """Oracle comparison with exact ownership.  The tolerance uses the contraction length of each
+    element's own group (`k`, when given, must be that length: it is only asserted, never trusted)."""
     want = oracle.grouped_mm(a, b, offs, out_dtype=out.dtype)
     got = out.cpu()
     # structure: exactly the owned elements are written
-    assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs"
-    oracle.assert_close(got, want, k)
+    assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs " + what
+    if k is not None and not (a.dim() == 2 and b.dim() == 2):
+        assert k == a.shape[-1]
+    oracle.assert_close_grouped(got, want, a, b, offs, what=what)
     if path is not None:
         assert K_.last_path() == path
 
@@ -97,7 +101,7 @@ def test_2d2d_bf16_empty_group_is_zero(path):
     a, b = rnd(gen, 16, 32), rnd(gen, 32, 24)
     with K_.forced_path(path):
         out = run_poisoned(K_.grouped_mm_2d2d, a, b, offs_of(sizes), (5, 16, 24), torch.bfloat16)
-    check(out, a, b, offs_of(sizes), 13)
+    check(out, a, b, offs_of(sizes))
     assert (out[1] == 0).all() and not torch.isnan(out.float()).any()
 
 
@@ -216,41 +220,6 @@ def test_all_layouts_all_variants_mfma(variant, a_col, b_col):
     check(out, a, b, offs, k, path="mfma")
 
 
-@pytest.mark.parametrize("a_col", [False, True])
-@pytest.mark.parametrize("b_col", [False, True])
-@pytest.mark.parametrize("variant", ["2d3d", "3d3d", "2d2d"])
-@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-def test_eight_wave_tile_all_layouts(variant, a_col, b_col, out_dtype):
-    """Tile configuration 2: the 256 x 256 tile computed by 8 waves (two per SIMD)."""
-    gen = torch.Generator().manual_seed(23)
-    sizes = [77, 0, 1, 330, 64, 200]  # sum 672
-    offs = offs_of(sizes)
-    G = len(sizes)
-    if variant == "2d3d":
-        a, b, shape, k, fn = rnd(gen, 672, 200), rnd(gen, G, 200, 520), (672, 520), 200, K_.grouped_mm_2d3d
-    elif variant == "3d3d":
-        a, b, shape, k, fn, offs = rnd(gen, 3, 304, 200), rnd(gen, 3, 200, 264), (3, 304, 264), 200, K_.grouped_mm_3d3d, None
-    else:
-        a, b, shape, k, fn = rnd(gen, 264, 672), rnd(gen, 672, 272), (G, 264, 272), 330, K_.grouped_mm_2d2d
-    ad, bd = a.to(DEV), b.to(DEV)
-    if a_col:
-        ad = ad.transpose(-2, -1).contiguous().transpose(-2, -1)
-    if b_col:
-        bd = bd.transpose(-2, -1).contiguous().transpose(-2, -1)
-    out = torch.full(shape, float("nan"), device=DEV, dtype=out_dtype)
-    with K_.forced_mfma_config(2):
-        if offs is None:
-            fn(ad, bd, out)
-        else:
-            fn(ad, bd, offs.to(DEV), out)
-        torch.cuda.synchronize()
-        assert K_._lib.load().gmm_last_mfma_config() == 2
-    want = oracle.grouped_mm(a, b, offs, out_dtype=out_dtype)
-    got = out.cpu()
-    assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs"
-    oracle.assert_close(got, want, k)
-
-
 @pytest.mark.parametrize("tall,shrt", [(256, 64), (256, 0), (128, 64), (128, 0)])
 @pytest.mark.parametrize("b_col", [False, True])
 def test_tile_heights_agree_bit_for_bit(tall, shrt, b_col):
@@ -362,7 +331,7 @@ def test_generic_family_on_the_matrix_cores(variant, a_col, b_col, dtype, tol):
     got = out.cpu()
     assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs"
     if tol is None:
-        oracle.assert_close(got, want, k)
+        oracle.assert_close_grouped(got, want, a, b, offs)
     else:
         owned = ~torch.isnan(want)
         torch.testing.assert_close(got[owned], want[owned], rtol=tol, atol=tol)
@@ -421,7 +390,7 @@ def test_random_shapes_all_variants(seed):
         want = oracle.grouped_mm(a, b, offs, out_dtype=out_dt)
         got = out.cpu()
         assert torch.equal(torch.isnan(got.float()), torch.isnan(want.float())), "ownership differs: " + what
-        oracle.assert_close(got, want, max(k, 1), what=what)
+        oracle.assert_close_grouped(got, want, a, b, offs, what=what)
 
 
 # ------------------------------------------------------------------ dtypes
@@ -517,7 +486,7 @@ def test_1023_groups_bf16_mfma_3d2d_and_2d2d():
     a2, b2 = rnd(gen, 16, k_total), rnd(gen, k_total, 24)
     with K_.forced_path("mfma"):
         out2 = run_poisoned(K_.grouped_mm_2d2d, a2, b2, offs, (1023, 16, 24), torch.bfloat16)
-    check(out2, a2, b2, offs, 3, path="mfma")
+    check(out2, a2, b2, offs, path="mfma")
 
 
 def test_fp32_epilogue_for_bf16_inputs_through_the_launcher():
@@ -639,15 +608,17 @@ def _sizes(golden_dir, key):
         return json.load(f)[key]
 
 
-def _sampled_check(out, a, b, offs_list, k, rows, cols=slice(None)):
-    """Oracle on a sample of rows of a big 2D x 3D result."""
-    ranges = oracle.group_ranges(offs_list)
-    for r in rows:
-        g = oracle.upper_bound(offs_list, r)
-        s, e = ranges[g]
-        assert s <= r < e
-        want = (a[r:r + 1].float() @ b[g].float()).to(out.dtype)
-        oracle.assert_close(out[r:r + 1].cpu(), want, k, what=f"row {r} group {g}")
+def _full_check_2d3d(out, a, b, offs_list, k, chunk=2048):
+    """The whole output against the oracle, group by group and in row chunks (bounded host memory)."""
+    got = out.cpu()
+    for g, (s, e) in enumerate(oracle.group_ranges(offs_list)):
+        if e == s:
+            continue
+        bg = b[g].float()
+        for r0 in range(s, e, chunk):
+            r1 = min(e, r0 + chunk)
+            want = (a[r0:r1].float() @ bg).to(out.dtype)
+            oracle.assert_close(got[r0:r1], want, k, what=f"rows {r0}:{r1} group {g}")
 
 
 def test_mixtral_up_projection_full_size(golden_dir):
@@ -657,13 +628,13 @@ def test_mixtral_up_projection_full_size(golden_dir):
     a = rnd(gen, 16384, 4096)
     b = rnd(torch.Generator().manual_seed(2), 8, 4096, 14336, scale=0.02)
     ad, bd = a.to(DEV), b.to(DEV)
-    out = grouped_mm(ad, bd, offs=offs.to(DEV))
+    out = torch.full((16384, 14336), float("nan"), device=DEV, dtype=torch.bfloat16)
+    K_.grouped_mm_2d3d(ad, bd, offs.to(DEV), out)
     assert K_.last_path() == "mfma"
-    ol = offs.tolist()
-    rows = sorted({0, 1, 255, 256, 16383, *ol[:-1], *[o - 1 for o in ol], *range(4800, 4830, 7), *range(0, 16384, 1999)})
-    _sampled_check(out, a, b, ol, 4096, rows)
-    # size-independent properties: splitting every group in two (same weights) and
-    # permuting the groups must reproduce the same rows bit for bit
+    assert not torch.isnan(out.float()).any()
+    _full_check_2d3d(out, a, b, offs.tolist(), 4096)     # every element, 1.9 TFLOP on the host
+    # size-independent properties: splitting every group in two (same weights) must reproduce the same
+    # rows bit for bit
     halves, idx = [], []
     for g, s in enumerate(sizes):
         halves += [s // 2, s - s // 2]
@@ -699,11 +670,13 @@ def test_batched_3d3d_full_size(b_col):
     bd = b.to(DEV)
     if b_col:
         bd = bd.transpose(1, 2).contiguous().transpose(1, 2)
-    out = grouped_mm(a.to(DEV), bd)
+    out = torch.full((32, 1024, 4096), float("nan"), device=DEV, dtype=torch.bfloat16)
+    K_.grouped_mm_3d3d(a.to(DEV), bd, out)
     assert K_.last_path() == "mfma"
-    for g in (0, 13, 31):
+    got = out.cpu()
+    for g in range(32):                                   # every batch, every element
         want = (a[g].float() @ b[g].float()).to(torch.bfloat16)
-        oracle.assert_close(out[g].cpu(), want, 1024, what=f"batch {g}")
+        oracle.assert_close(got[g], want, 1024, what=f"batch {g}")
 
 
 def test_k_grouped_weight_gradient_full_size(golden_dir):
@@ -716,12 +689,11 @@ def test_k_grouped_weight_gradient_full_size(golden_dir):
     K_.grouped_mm_2d2d(ad, bd, offs.to(DEV), out)
     assert K_.last_path() == "mfma"
     assert not torch.isnan(out).any()
-    rngs = oracle.group_ranges(offs.tolist())
-    for g in (0, 3, 7):
-        s, e = rngs[g]
-        rows = [0, 255, 256, 4095]
-        want = a[rows][:, s:e].float() @ b[s:e].float()
-        torch.testing.assert_close(out[g][rows].cpu(), want, rtol=1.6e-2, atol=1e-2 * ((e - s) / 64) ** 0.5)
-    # the groups partition K: their sum is the plain product (checked on a row band)
-    total = out[:, :64].sum(0).cpu()
-    torch.testing.assert_close(total, a[:64].float() @ b.float(), rtol=1.6e-2, atol=0.5)
+    total = torch.zeros(4096, 14336)
+    for g, (s, e) in enumerate(oracle.group_ranges(offs.tolist())):   # every group, every element
+        got = out[g].cpu()
+        want = a[:, s:e].float() @ b[s:e].float()
+        oracle.assert_close(got, want, e - s, what=f"group {g}")
+        total += got
+    # the groups partition K: their sum is the plain product
+    torch.testing.assert_close(total, a.float() @ b.float(), rtol=1.6e-2, atol=1e-2 * (16384 / 64) ** 0.5)
