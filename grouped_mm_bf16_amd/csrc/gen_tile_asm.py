@@ -34,12 +34,11 @@ wave, 4 x 4 MFMA blocks of 32 x 32); variants for 128 x 256 and 64 x 256 tiles
   * one s_barrier per K tile, placed after step 2 so that step 3's MFMAs run
     while the barrier's stragglers arrive and the first fragments of the next
     tile are fetched under them;
-  * epilogue, 16-bit output: the MFMA operands are swapped so a lane owns 4
-    consecutive columns, packs them (v_cvt_pk_bf16_f32), stages the wave's block
-    in LDS and writes 16 bytes per lane, 256 contiguous bytes per row; a chunk
-    that a group boundary cuts (jagged columns) goes out as 2-byte stores;
-    fp32: each accumulator register goes out as one dword store, 128 contiguous
-    bytes per row.
+  * epilogue: the MFMA operands are swapped so a lane owns 4 consecutive columns;
+    it packs them (v_cvt_pk_bf16_f32; fp32 goes as it is), stages the wave's block
+    in LDS and writes 16 bytes per lane: 256 contiguous bytes per row (512 for
+    fp32); a chunk that a group boundary cuts (jagged columns) goes out element
+    by element.
 
 Registers:
   a[0:255]     accumulators, block (i, j) at a[(4 i + j) 16 ...]
@@ -54,14 +53,10 @@ import sys
 COPY_SCHEDULE = (8, 8, 0, 0)
 
 PITCH = 272           # bytes per staged row of 128 bf16 (256 + 16: shifts banks per row)
+PITCH32 = 528         # ... of 128 fp32 (512 + 16)
 TR_BLOCK = 1088       # two k rows of 512 bytes + 64 bytes pad
 KC_STAGE = 256 * 64 * 2
 TR_STAGE = 32 * TR_BLOCK
-# 256-row tile: K is walked in half tiles of 32 through a ring of four LDS slots per operand
-RING = 4
-RING_ENABLED = False
-RING_KC_SLOT = 256 * 32 * 2      # [row][32 k]: 64-byte rows, chunks XOR-swizzled by (row >> 2) & 3
-RING_TR_SLOT = 16 * TR_BLOCK     # [k][256] in 16 blocks of two k rows
 STAGE_BYTES = 4 * 128 * PITCH
 
 # ---- fixed register map: one wave per SIMD (128 x 128 per wave, 256 accumulators), the wave owns all 512
@@ -127,15 +122,6 @@ class Variant:
         self.a_stage = TR_STAGE if a_tr else (64 * tm * 128 if self.stages == 3 else KC_STAGE)
         self.b_stage = TR_STAGE if b_tr else KC_STAGE
         self.b_base = self.stages * self.a_stage   # LDS offset of B buffer 0
-        self.ring = RING_ENABLED and tm == 4
-        if self.ring:
-            self.na = self.nb = 4                # copies per wave and half tile, per operand
-            self.ncopy = 8
-            self.stages = RING
-            self.a_stage = RING_TR_SLOT if a_tr else RING_KC_SLOT
-            self.b_stage = RING_TR_SLOT if b_tr else RING_KC_SLOT
-            self.b_base = RING * self.a_stage
-        self.swap = not out_f32                  # bf16: lanes own 4 consecutive columns
         self.name = "%s%s_%s_%s_m%d" % ("t" if a_tr else "k", "t" if b_tr else "k", self.dt, "f32" if out_f32 else self.dt, 64 * tm)
 
     def acc(self, i, j):
@@ -152,20 +138,17 @@ class Variant:
         ):
             # two buffers: the buffer is an immediate offset; three: one address register per buffer and
             # step (set up by the prologue), because the offsets no longer fit the 16-bit immediate
-            if self.stages == 2 or self.ring:
+            if self.stages == 2:
                 reg, boff = (vaddr + s if not tr else vaddr), buf * stage
             else:
                 reg, boff = (vbuf + 4 * buf + s if not tr else vbuf + 4 * buf), 0
-            sub = 2048 if self.ring else 4096
             for x in range(nblk):
                 d = vbase + 4 * x
                 if not tr:
-                    # address register per step; sub-tiles are 32 rows = 4096 bytes apart (2048 in the ring's 64-byte rows)
-                    assert boff + x * sub < 65536
-                    blocks[(op, x)] = ["ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(reg), boff + x * sub)]
+                    # address register per step; sub-tiles are 32 rows = 4096 bytes apart
+                    blocks[(op, x)] = ["ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(reg), boff + x * 4096)]
                 else:
                     o = boff + s * 8 * TR_BLOCK + x * 64
-                    assert o + 512 < 65536
                     blocks[(op, x)] = ["ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d, 2), vr(reg), o),
                                        "ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d + 2, 2), vr(reg), o + 512)]
         self.read_order = [("A", 0)] + [("B", x) for x in range(self.tn)] + [("A", x) for x in range(1, self.tm)]
@@ -196,8 +179,8 @@ class Variant:
                 a = vr(V_AF[st] + 4 * i, 4)
                 b = vr(V_BF[st] + 4 * j, 4)
                 c = "a[%d:%d]" % (self.acc(i, j), self.acc(i, j) + 15)
-                x, y = (b, a) if self.swap else (a, b)
-                out.append("v_mfma_f32_32x32x16_%s %s, %s, %s, %s" % (self.dt, c, x, y, c))
+                # operands swapped: the result block is transposed, a lane owns 4 consecutive columns of a row
+                out.append("v_mfma_f32_32x32x16_%s %s, %s, %s, %s" % (self.dt, c, b, a, c))
         return out
 
     # -- copy instruction n (0..15) of a K tile into buffer buf.
@@ -205,9 +188,8 @@ class Variant:
     # s_ka / s_kb: SGPRs with the tile's byte offsets along K for A and B.  which: "head" or "loop".
     def dma(self, n, buf, which, s_tail, s_oob, s_ka, s_kb, tmp):
         out = []
-        # ring: B's copies go first (B is the operand that streams from HBM in the MoE shapes)
-        is_a = n >= self.nb if self.ring else n < self.na
-        i = (n - self.nb if is_a else n) if self.ring else (n if is_a else n - self.na)
+        is_a = n < self.na
+        i = n if is_a else n - self.na
         tr = self.a_tr if is_a else self.b_tr
         stage = self.a_stage if is_a else self.b_stage
         lbase = 0 if is_a else self.b_base
@@ -247,8 +229,7 @@ def m0_gaps(lines):
 
 def fixup(e, v, which, buf):
     """Zero the k elements outside the group's range in one 16-byte chunk per row (row = thread id) of
-    every operand that is contiguous along K.  which: 0 = first chunk of K tile 0, 1 = last chunk.
-    buf: LDS buffer of the tile (ring: the addresses already point into the right slot, pass 0)."""
+    every operand that is contiguous along K.  which: 0 = first chunk of K tile 0, 1 = last chunk."""
     for is_a in (True, False):
         tr = v.a_tr if is_a else v.b_tr
         if tr:
@@ -309,8 +290,8 @@ def interleave(e, mfmas, side_groups, need=None, prev_total=0):
         e(ins)
 
 
-def gen_classic_main(v, e, L):
-    """Prologue and K loop of the 128- and 64-row tiles: K tiles of 64 through three LDS buffers."""
+def gen_main(v, e, L):
+    """Prologue and K loop: K tiles of 64 through two (256-row tile) or three LDS buffers."""
     sT = S_T
     # temporaries
     s_kt, s_t1 = sT + 0, sT + 1
@@ -475,270 +456,104 @@ def gen_classic_main(v, e, L):
     e.label("L_done_%s" % L)
 
 
-def merge_side(reads, copies):
-    """One list of side groups: the copy groups spread evenly among the fragment reads."""
-    total, nc = len(reads) + len(copies), len(copies)
-    at = {(j + 1) * total // nc - 1: j for j in range(nc)} if nc else {}
-    out, r = [], iter(reads)
-    for k in range(total):
-        out.append(copies[at[k]] if k in at else next(r))
-    return out
-
-
-def gen_ring_main(v, e, L):
-    """Prologue and K loop of the 256-row tile.  K is walked in half tiles of 32 (two k16 steps, 32 MFMAs
-    per wave) through a ring of four LDS slots per operand: while half h is multiplied, halves h + 1 and
-    h + 2 are in flight or landed and the copies of half h + 3 are issued, four per step, into the slot
-    that half h - 1 left at the last barrier.  Every copy therefore has two to three half tiles (2000 to
-    3000 cycles) to land, and the copies are spread evenly over the MFMAs instead of coming in bursts.
-    One barrier per half, after step 0: it publishes half h + 1 and releases the slot of half h."""
-    sT = S_T
-    s_h, s_t1 = sT + 0, sT + 1
-    s_ka, s_kb = sT + 2, sT + 3          # K offsets of the half whose copies are being issued
-    s_tail, s_oob = sT + 6, sT + 8       # pairs
-    s_last = sT + 14                     # nh - 1
-    s_zero = sT + 15
-    s_flags = sT + 18
-    s_waveA, s_waveB = sT + 20, sT + 21
-    NC = v.ncopy
-
-    def half_masks(s_half):
-        # tail mask: half == nh - 1 ; oob mask: half >= nh
-        e("s_cmp_eq_u32 %s, %s" % (sr(s_half), sr(s_last)))
-        e("s_cselect_b64 %s, -1, 0" % sr(s_tail, 2))
-        e("s_cmp_ge_u32 %s, %s" % (sr(s_half), sr(S_NK)))
-        e("s_cselect_b64 %s, -1, 0" % sr(s_oob, 2))
-
-    e("; ---- prologue (%s, ring)" % v.name)
-    e("v_mov_b32 %s, 0x80000000" % vr(V_OOB))
-    # s[S_SPARE] = wave id | flags << 8 (bit 0: first chunk of the k range is partial, bit 1: last chunk, bit 2: partial output chunks)
-    e("s_lshr_b32 %s, %s, 8" % (sr(s_flags), sr(S_SPARE)))
-    e("s_and_b32 %s, %s, 0xff" % (sr(sT + 19), sr(S_SPARE)))
-    e("s_sub_u32 %s, %s, 1" % (sr(s_last), sr(S_NK)))
-    e("s_mov_b32 %s, 0" % sr(s_zero))
-    e("s_mul_i32 %s, %s, %d" % (sr(s_waveA), sr(sT + 19), v.na * (TR_BLOCK if v.a_tr else 1024)))
-    e("s_add_u32 %s, %s, %s" % (sr(s_waveA), sr(s_waveA), sr(S_LDS)))
-    e("s_mul_i32 %s, %s, %d" % (sr(s_waveB), sr(sT + 19), v.nb * (TR_BLOCK if v.b_tr else 1024)))
-    e("s_add_u32 %s, %s, %s" % (sr(s_waveB), sr(s_waveB), sr(S_LDS)))
-    # halves 0, 1, 2 -> slots 0, 1, 2
-    for n in range(NC):
-        for ins in m0_gaps(v.dma(n, 0, "head", 0, 0, s_zero, s_zero, V_TMP)):
-            e(ins)
-    for hx in (1, 2):
-        e("s_mov_b32 %s, %d" % (sr(s_t1), hx))
-        half_masks(s_t1)
-        e("s_mul_i32 %s, %s, %d" % (sr(s_ka), sr(S_ASTEP), hx))
-        e("s_mul_i32 %s, %s, %d" % (sr(s_kb), sr(S_BSTEP), hx))
-        for n in range(NC):
-            for ins in m0_gaps(v.dma(n, hx, "loop", s_tail, s_oob, s_ka, s_kb, V_TMP + (n % 8))):
-                e(ins)
-    for r in range(16 * v.tm * v.tn):
-        e("v_accvgpr_write_b32 a%d, 0" % r)
-    e("s_waitcnt vmcnt(%d)" % (2 * NC))
-    e("s_barrier")
-    if not (v.a_tr and v.b_tr):
-        # partial first / last chunk of a jagged k range (half 0 is also the last half when nh == 1)
-        e("s_and_b32 %s, %s, 3" % (sr(s_t1), sr(s_flags)))
-        e("s_cmp_eq_u32 %s, 0" % sr(s_t1))
-        e("s_cbranch_scc1 L_nofix0_%s" % L)
-        e("s_bitcmp1_b32 %s, 0" % sr(s_flags))
-        e("s_cbranch_scc0 L_nohead_%s" % L)
-        fixup(e, v, 0, 0)
-        e("s_waitcnt lgkmcnt(0)")
-        e.label("L_nohead_%s" % L)
-        e("s_bitcmp1_b32 %s, 1" % sr(s_flags))
-        e("s_cbranch_scc0 L_notail0_%s" % L)
-        e("s_cmp_eq_u32 %s, 1" % sr(S_NK))
-        e("s_cbranch_scc0 L_notail0_%s" % L)
-        fixup(e, v, 1, 0)
-        e.label("L_notail0_%s" % L)
-        e("s_waitcnt lgkmcnt(0)")
-        e("s_barrier")
-        e.label("L_nofix0_%s" % L)
-    for ins in v.frag_reads(0, 0, 0):
-        e(ins)
-    e("s_mov_b32 %s, 0" % sr(s_h))
-    e("s_cmp_eq_u32 %s, 0" % sr(S_NK))
-    e("s_cbranch_scc1 L_done_%s" % L)
-
-    need, nreads = v.read_need()
-
-    def half(slot, fast):
-        # on entry: fragments of step 0 in set 0 (in flight); halves h + 1, h + 2 in flight or landed
-        which = "fast" if fast else "loop"
-        e("; ---- half tile on slot %d%s" % (slot, " (interior)" if fast else ""))
-        e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_h), RING - 1))
-        if not fast:
-            half_masks(s_t1)
-        e("s_mul_i32 %s, %s, %s" % (sr(s_ka), sr(s_t1), sr(S_ASTEP)))
-        e("s_mul_i32 %s, %s, %s" % (sr(s_kb), sr(s_t1), sr(S_BSTEP)))
-        nxt = (slot + 1) % RING            # slot of half h + 1
-        dst = (slot + RING - 1) % RING     # slot of half h + 3 (= of half h - 1)
-        copies = [v.dma(n, dst, which, s_tail, s_oob, s_ka, s_kb, V_TMP + (n % 8)) for n in range(NC)]
-        # step 0: MFMA set 0, read step 1 -> set 1, first half of the copies
-        side = merge_side([[x] for x in v.frag_reads(slot, 1, 1)], copies[:NC // 2])
-        interleave(e, v.mfmas(0), side, need, nreads)
-        # half h + 1 has landed for this wave (the copies of halves h + 2 and h + 3 stay in flight); after
-        # the barrier it has for all waves, and everyone is done reading this slot
-        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % (NC + NC // 2))
-        e("s_barrier")
-        if not (v.a_tr and v.b_tr) and not fast:
-            # the half that has just landed is the last one and its last chunk is partial
-            e("s_add_u32 %s, %s, 1" % (sr(s_t1), sr(s_h)))
-            e("s_cmp_eq_u32 %s, %s" % (sr(s_t1), sr(s_last)))
-            e("s_cbranch_scc0 L_nofix%d_%s" % (slot + 1, L))
-            e("s_bitcmp1_b32 %s, 1" % sr(s_flags))
-            e("s_cbranch_scc0 L_nofix%d_%s" % (slot + 1, L))
-            fixup(e, v, 1, 0)
-            e("s_waitcnt lgkmcnt(0)")
-            e("s_barrier")
-            e.label("L_nofix%d_%s" % (slot + 1, L))
-        # step 1: MFMA set 1, read step 0 of the next half -> set 0, the other copies
-        side = merge_side([[x] for x in v.frag_reads(nxt, 0, 0)], copies[NC // 2:])
-        interleave(e, v.mfmas(1), side)
-        e("s_add_u32 %s, %s, 1" % (sr(s_h), sr(s_h)))
-
-    def half_both(slot):
-        e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_h), RING - 1))
-        e("s_cmp_lt_u32 %s, %s" % (sr(s_t1), sr(s_last)))
-        e("s_cbranch_scc0 L_slow%d_%s" % (slot, L))
-        half(slot, True)
-        e("s_branch L_join%d_%s" % (slot, L))
-        e.label("L_slow%d_%s" % (slot, L))
-        half(slot, False)
-        e.label("L_join%d_%s" % (slot, L))
-
-    e.label("L_loop_%s" % L)
-    for slot in range(RING - 1):
-        half_both(slot)
-        e("s_cmp_ge_u32 %s, %s" % (sr(s_h), sr(S_NK)))
-        e("s_cbranch_scc1 L_done_%s" % L)
-    half_both(RING - 1)
-    e("s_cmp_lt_u32 %s, %s" % (sr(s_h), sr(S_NK)))
-    e("s_cbranch_scc1 L_loop_%s" % L)
-    e.label("L_done_%s" % L)
-
-
 def gen_variant(v):
     e = Emit()
     L = "%s_%%=" % v.name  # unique label suffix per asm instance
-    if v.ring:
-        gen_ring_main(v, e, L)
-    else:
-        gen_classic_main(v, e, L)
+    gen_main(v, e, L)
     gen_epilogue(v, e, L)
     return e
 
 
 def gen_epilogue(v, e, L):
+    """Accumulators -> output.  The MFMA operands are swapped, so a lane owns 4 consecutive columns of a
+    row: acc block (i, j), register 4 q + r  ->  C[m = 32 i + lane % 32][n = 32 j + 8 q + 4 (lane / 32) + r].
+    The wave stages its block in LDS (rows padded to `pitch` bytes; `ipp` MFMA block rows per pass: all of
+    them for a 16-bit output, one for fp32, whose rows are twice as long) and reads it back so that each lane
+    holds 16 consecutive bytes of a row: every store instruction writes whole rows of the wave's 128 columns
+    (256 contiguous bytes of 4 rows, or 512 contiguous bytes of 2 rows for fp32).
+    v[V_EPI + 0] = stage write address, v[V_EPI + 1] = stage read address,
+    v[V_EPI + 2] = store offset of the lane's chunk in read-back instruction 0 (or out-of-range when the
+                   lane's columns are not all valid), v[V_EPI + 3] = its row - row_lo, valid iff (unsigned) < S_ROWCNT,
+    v[V_EPI2 + 0] = that store offset whatever the validity, v[V_EPI2 + 1] = mask of valid elements of a
+                   chunk that a group boundary cuts (tile flag bit 2): those go out element by element."""
     e("; ---- epilogue")
-    t = V_TMP
     e("s_waitcnt vmcnt(0) lgkmcnt(0)")
     e("s_nop 15")
     e("s_nop 15")
     e("s_barrier")
-    if not v.out_f32:
-        # acc block (i, j), register 4 q + r  ->  C[m = 32 i + lane % 32][n = 32 j + 8 q + 4 (lane / 32) + r]
-        # The wave stages its block in LDS (rows padded to `pitch` bytes), `ipp` MFMA block rows per pass, and
-        # reads it back so that each lane holds 16 consecutive bytes of a row.
-        # v[V_EPI + 2] = store offset of the lane's row in read-back instruction 0 (or OOB when the lane's
-        #                columns are invalid); v[V_EPI + 3] = that row - row_lo, valid iff (unsigned) < S_ROWCNT
-        t = V_TMP
-        pitch = PITCH
-        ipp = v.tm
-        rpi = 16 // v.tn          # rows per read-back instruction (64 lanes x 16 bytes over rows of 32 tn columns)
-        depth = 4
-        regs = [t + 4 * x for x in range(depth)]          # read-back data, 4 registers each
-        voff, vrow, vsel = t + 24, t + 25, t + 26
-        e("v_mov_b32 %s, %s" % (vr(voff), vr(V_EPI + 2)))
-        e("v_mov_b32 %s, %s" % (vr(vrow), vr(V_EPI + 3)))
-        partial = True
-        if partial:
-            # A group boundary that is not a multiple of 8 columns leaves 16-byte chunks of which only some
-            # elements belong to this tile (flag bit 2 of the tile): those go out as 2-byte stores.
-            # eoff[e] = 2 e if element e of the lane's chunk is valid, else the out-of-range offset
-            eoff, vpoff, vtmp = t + 27, t + 35, t + 36
-            e("s_bitcmp1_b32 %s, 2" % sr(S_T + 18))
-            e("s_cbranch_scc0 L_nopart_setup_%s" % L)
-            e("v_mov_b32 %s, %s" % (vr(vpoff), vr(V_EPI2)))
-            for el in range(8):
-                e("v_bfe_u32 %s, %s, %d, 1" % (vr(vtmp), vr(V_EPI2 + 1), el))
-                e("v_cmp_ne_u32 vcc, 0, %s" % vr(vtmp))
-                e("v_mov_b32 %s, %d" % (vr(vtmp), 2 * el))
-                e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(eoff + el), vr(V_OOB), vr(vtmp)))
-            e.label("L_nopart_setup_%s" % L)
-        nstore = 0
-        for p0 in range(0, v.tm, ipp):
-            k = 0
-            for il in range(min(ipp, v.tm - p0)):
-                i = p0 + il
-                for j in range(v.tn):
-                    for q in range(4):
-                        b = t + 6 * (k % 4)
-                        k += 1
-                        a0 = v.acc(i, j) + 4 * q
-                        for r in range(4):
-                            e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), a0 + r))
+    t = V_TMP
+    f32 = v.out_f32
+    esz = 4 if f32 else 2
+    nel = 16 // esz                       # elements of a 16-byte chunk
+    pitch = PITCH32 if f32 else PITCH
+    ipp = 1 if f32 else v.tm              # MFMA block rows per pass
+    rpi = 1024 // (32 * v.tn * esz)       # rows per read-back instruction (64 lanes x 16 bytes)
+    depth = 4
+    regs = [t + 4 * x for x in range(depth)]          # read-back data, 4 registers each
+    voff, vrow, vsel = t + 24, t + 25, t + 26
+    eoff, vpoff, vtmp = t + 27, t + 35, t + 36
+    e("v_mov_b32 %s, %s" % (vr(voff), vr(V_EPI + 2)))
+    e("v_mov_b32 %s, %s" % (vr(vrow), vr(V_EPI + 3)))
+    # eoff[el] = byte offset of element el of the lane's chunk if it is valid, else the out-of-range offset
+    e("s_bitcmp1_b32 %s, 2" % sr(S_T + 18))
+    e("s_cbranch_scc0 L_nopart_setup_%s" % L)
+    e("v_mov_b32 %s, %s" % (vr(vpoff), vr(V_EPI2)))
+    for el in range(nel):
+        e("v_bfe_u32 %s, %s, %d, 1" % (vr(vtmp), vr(V_EPI2 + 1), el))
+        e("v_cmp_ne_u32 vcc, 0, %s" % vr(vtmp))
+        e("v_mov_b32 %s, %d" % (vr(vtmp), esz * el))
+        e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(eoff + el), vr(V_OOB), vr(vtmp)))
+    e.label("L_nopart_setup_%s" % L)
+    nstore = 0
+    for p0 in range(0, v.tm, ipp):
+        k = 0
+        for il in range(min(ipp, v.tm - p0)):
+            i = p0 + il
+            for j in range(v.tn):
+                for q in range(4):
+                    b = t + 6 * (k % 4)
+                    k += 1
+                    a0 = v.acc(i, j) + 4 * q
+                    for r in range(4):
+                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), a0 + r))
+                    if f32:
+                        e("ds_write_b128 %s, %s offset:%d" % (vr(V_EPI), vr(b, 4), (32 * il) * pitch + (32 * j + 8 * q) * 4))
+                    else:
                         e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 4), vr(b), vr(b + 1)))
                         e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 5), vr(b + 2), vr(b + 3)))
                         e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 4, 2), (32 * il) * pitch + (32 * j + 8 * q) * 2))
-            e("s_waitcnt lgkmcnt(0)")
-            nrb = min(ipp, v.tm - p0) * 32 // rpi   # read-back instructions of this pass
-            for r in range(min(depth, nrb)):
-                e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r], 4), vr(V_EPI + 1), r * rpi * pitch))
-            for r in range(nrb):
-                e("s_waitcnt lgkmcnt(%d)" % min(depth - 1, nrb - 1 - r))
-                e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
-                e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vsel), vr(V_OOB), vr(voff)))
-                e("buffer_store_dwordx4 %s, %s, %s, 0 offen" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
-                if partial:
-                    e("s_bitcmp1_b32 %s, 2" % sr(S_T + 18))
-                    e("s_cbranch_scc0 L_nopart%d_%s" % (nstore, L))
-                    for el in range(8):
-                        e("v_add_u32 %s, %s, %s" % (vr(vtmp), vr(eoff + el), vr(vpoff)))
-                        e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vtmp + 1 + el % 2), vr(V_OOB), vr(vtmp)))
-                        e("buffer_store_short%s %s, %s, %s, 0 offen" % ("_d16_hi" if el % 2 else "", vr(regs[r % depth] + el // 2),
-                                                                         vr(vtmp + 1 + el % 2), sr(S_RC, 4)))
-                    e("v_add_u32 %s, %s, %s" % (vr(vpoff), sr(S_CSTEP), vr(vpoff)))
-                    e.label("L_nopart%d_%s" % (nstore, L))
-                    nstore += 1
-                if r + depth < nrb:
-                    # the store above must have read its data before the register is reloaded
-                    e("s_nop 0")
-                    e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r % depth], 4), vr(V_EPI + 1), (r + depth) * rpi * pitch))
-                e("v_add_u32 %s, %s, %s" % (vr(voff), sr(S_CSTEP), vr(voff)))
-                e("v_add_u32 %s, %d, %s" % (vr(vrow), rpi, vr(vrow)))
-            if p0 + ipp < v.tm:
-                # the next pass overwrites the staging area and the read-back registers: reads are done
-                # (lgkmcnt 0 above); the last stores must have fetched their data
-                e("s_nop 4")
-    else:
-        # acc block (i, j), register 4 q + r -> C[m = 32 i + 8 q + 4 (lane / 32) + r][n = 32 j + lane % 32]
-        # v[V_EPI + 2] = store offset of (row 4 (lane / 32), col lane % 32); v[V_EPI + 3] = 4 (lane / 32) - row_lo
-        # column validity of block j: lane mask pairs s[S_T + 24 + 2 j]
-        t = V_TMP
-        voff, vrow, vsel = t + 16, t + 17, t + 18
-        for j in range(v.tn):
-            e("v_add_u32 %s, %d, %s" % (vr(t + 19), 32 * j, vr(V_EPI + 1)))   # V_EPI + 1 = lane % 32 (column in block)
-            e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_NVALID), vr(t + 19)))
-            e("s_mov_b64 %s, vcc" % sr(S_T + 24 + 2 * j, 2))
-        k = 0
-        e("s_mov_b32 %s, 0" % sr(S_T + 16))   # running row offset in bytes
-        for i in range(v.tm):
-            for q in range(4):
-                for r in range(4):
-                    row = 32 * i + 8 * q + r
-                    e("v_add_u32 %s, %d, %s" % (vr(vrow), row, vr(V_EPI + 3)))
-                    e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
-                    e("s_mov_b64 %s, vcc" % sr(S_T + 32, 2))
-                    e("s_mul_i32 %s, %s, %d" % (sr(S_T + 16), sr(S_CSTEP), row))
-                    for j in range(v.tn):
-                        b = t + (k % 8)
-                        k += 1
-                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b), v.acc(i, j) + 4 * q + r))
-                        e("s_and_b64 vcc, %s, %s" % (sr(S_T + 32, 2), sr(S_T + 24 + 2 * j, 2)))
-                        e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(t + 8 + (k % 8)), vr(V_OOB), vr(V_EPI + 2)))
-                        e("buffer_store_dword %s, %s, %s, %s offen offset:%d" % (vr(b), vr(t + 8 + (k % 8)), sr(S_RC, 4), sr(S_T + 16), 128 * j))
+        e("s_waitcnt lgkmcnt(0)")
+        nrb = min(ipp, v.tm - p0) * 32 // rpi   # read-back instructions of this pass
+        for r in range(min(depth, nrb)):
+            e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r], 4), vr(V_EPI + 1), r * rpi * pitch))
+        for r in range(nrb):
+            e("s_waitcnt lgkmcnt(%d)" % min(depth - 1, nrb - 1 - r))
+            e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
+            e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vsel), vr(V_OOB), vr(voff)))
+            e("buffer_store_dwordx4 %s, %s, %s, 0 offen" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
+            e("s_bitcmp1_b32 %s, 2" % sr(S_T + 18))
+            e("s_cbranch_scc0 L_nopart%d_%s" % (nstore, L))
+            for el in range(nel):
+                e("v_add_u32 %s, %s, %s" % (vr(vtmp), vr(eoff + el), vr(vpoff)))
+                e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vtmp + 1 + el % 2), vr(V_OOB), vr(vtmp)))
+                if f32:
+                    e("buffer_store_dword %s, %s, %s, 0 offen" % (vr(regs[r % depth] + el), vr(vtmp + 1 + el % 2), sr(S_RC, 4)))
+                else:
+                    e("buffer_store_short%s %s, %s, %s, 0 offen" % ("_d16_hi" if el % 2 else "", vr(regs[r % depth] + el // 2),
+                                                                     vr(vtmp + 1 + el % 2), sr(S_RC, 4)))
+            e("v_add_u32 %s, %s, %s" % (vr(vpoff), sr(S_CSTEP), vr(vpoff)))
+            e.label("L_nopart%d_%s" % (nstore, L))
+            nstore += 1
+            if r + depth < nrb:
+                # the store above must have read its data before the register is reloaded
+                e("s_nop 0")
+                e("ds_read_b128 %s, %s offset:%d" % (vr(regs[r % depth], 4), vr(V_EPI + 1), (r + depth) * rpi * pitch))
+            e("v_add_u32 %s, %s, %s" % (vr(voff), sr(S_CSTEP), vr(voff)))
+            e("v_add_u32 %s, %d, %s" % (vr(vrow), rpi, vr(vrow)))
+        if p0 + ipp < v.tm:
+            # the next pass overwrites the staging area and the read-back registers: reads are done
+            # (lgkmcnt 0 above); the last stores must have fetched their data
+            e("s_nop 4")
     e("s_waitcnt lgkmcnt(0)")
     e("s_barrier")
 
@@ -756,6 +571,7 @@ def main():
     out.append("// Generated by gen_tile_asm.py -- do not edit.")
     out.append("// Per-tile main loop + epilogue in gfx950 assembly, one function per operand-layout / output variant.")
     out.append("#define GMM_TILE_PITCH %d" % PITCH)
+    out.append("#define GMM_TILE_PITCH32 %d" % PITCH32)
     out.append("#define GMM_TILE_TR_BLOCK %d" % TR_BLOCK)
     out.append("#define GMM_TILE_KC_STAGE %d" % KC_STAGE)
     out.append("#define GMM_TILE_TR_STAGE %d" % TR_STAGE)

@@ -74,10 +74,13 @@ bool asm_tile_eligible(const Problem& pr, const GmmLayout& lay) {
   // a transposed-layout operand is addressed from its first k row: the whole slice must fit 31 bits
   if (!lay.a_kc && int64_t(p.K) * lda * 2 >= (int64_t(1) << 31)) return false;
   if (!lay.b_kc && int64_t(p.K) * ldb * 2 >= (int64_t(1) << 31)) return false;
+  // the epilogue stores 16-byte chunks of a row
+  if (!aligned16(p.c)) return false;
   if (pr.out_dtype != GMM_DT_F32) {
-    if (!aligned16(p.c) || !mult8(p.c_sm) || !mult8(p.c_sg) || !mult8(p.N)) return false;
-  } else if (ldc >= ld_max / 2) {
-    return false;   // 255 rows of 4-byte elements must stay below 2^31 bytes from the tile's origin
+    if (!mult8(p.c_sm) || !mult8(p.c_sg) || !mult8(p.N)) return false;
+  } else {
+    if ((p.c_sm & 3) || (p.c_sg & 3)) return false;
+    if (ldc >= ld_max / 2) return false;   // 255 rows of 4-byte elements must stay below 2^31 bytes from the tile's origin
   }
   return true;
 }

@@ -92,7 +92,9 @@ __device__ __forceinline__ void gmm_scan_table(int32_t* cum) {
   }
 }
 
-// Returns the total number of tiles; total_tall gets the number of tall ones.
+// Returns the total number of tiles; total_tall gets the number of tall ones (they come first in the launch
+// order: the workgroups of all XCDs then work on tiles of one height in every round and stay in step, which
+// keeps the operand panels they share in the Infinity Cache).
 template <int NT>
 __device__ __forceinline__ int gmm_build_tile_table2(const GmmParams& p, int bn, int32_t* cum_tall, int32_t* cum_short,
                                                      int& total_tall) {

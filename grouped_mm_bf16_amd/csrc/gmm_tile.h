@@ -20,7 +20,7 @@ struct GmmTileRegs {
   gmm_v4i fix;                 // LDS addresses of this thread's row in the first / last k chunk (A, A, B, B)
   gmm_v8i masks;               // keep-masks of the first and of the last 16-byte k chunk
   gmm_v4i rsrc_a, rsrc_b, rsrc_c;
-  gmm_v8i scal;                // nk, a_step, b_step, lds_base, row_cnt, c_step, n_valid, wave
+  gmm_v8i scal;                // nk, a_step, b_step, lds_base, row_cnt, c_step, (unused), wave | flags << 8
 };
 
 // TM = MFMA block rows per wave: the tile is 64 * TM rows (256, 128 or 64) by 256 columns.
@@ -49,7 +49,10 @@ template <int A_TR, int B_TR, int TM>
 constexpr int gmm_tile_lds_bytes() {
   using L = GmmTileLayout<A_TR, TM>;
   constexpr int pipe = L::b_base + L::stages * (B_TR ? GMM_TILE_TR_STAGE : GMM_TILE_KC_STAGE);
-  constexpr int staging = 64 * TM * 2 * GMM_TILE_PITCH;
+  // staging of the epilogue: one padded row of 256 columns per tile row (16-bit output), or 32 rows of
+  // 128 fp32 columns per wave and pass; both are below the pipeline buffers of every tile height
+  constexpr int staging16 = 64 * TM * 2 * GMM_TILE_PITCH, staging32 = 4 * 32 * GMM_TILE_PITCH32;
+  constexpr int staging = staging16 > staging32 ? staging16 : staging32;
   return pipe > staging ? pipe : staging;
 }
 
@@ -154,36 +157,33 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
       r.rb_addr[s] = lds_base + B_BASE + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wn * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
     }
   }
-  int c_step, n_valid = 0, partial = 0;
-  r.epi2[0] = 0;
-  r.epi2[1] = 0;
-  if (!OUT_F32) {
-    const int row_t = wm * WROWS + (lane >> 4), col_t = wn * 128 + (lane & 15) * 8;
-    r.epi[0] = lds_base + wave * (WROWS * GMM_TILE_PITCH) + (lane & 31) * GMM_TILE_PITCH + 8 * (lane >> 5);
-    r.epi[1] = lds_base + wave * (WROWS * GMM_TILE_PITCH) + (lane >> 4) * GMM_TILE_PITCH + (lane & 15) * 16;
-    // the lane's 8 columns: all valid -> one 16-byte store; some valid (a group boundary that is not a
-    // multiple of 8 columns) -> element stores under the mask; none -> nothing
+  // Epilogue: the wave stages its block in LDS and reads it back row by row, 16 bytes per lane (see
+  // gen_tile_asm.py).  ESZ bytes per element: a lane's chunk is NEL = 16 / ESZ columns, a row of the wave's
+  // 128 columns takes LPR lanes, a read-back instruction covers 64 / LPR rows.
+  constexpr int ESZ = OUT_F32 ? 4 : 2, NEL = 16 / ESZ, LPR = 128 / NEL;
+  constexpr int EPITCH = OUT_F32 ? GMM_TILE_PITCH32 : GMM_TILE_PITCH;
+  constexpr int STAGE_ROWS = OUT_F32 ? 32 : WROWS;        // rows a wave stages per pass
+  int partial = 0;
+  {
+    const int row_t = wm * WROWS + lane / LPR, col_t = wn * 128 + (lane % LPR) * NEL;
+    const unsigned stage = lds_base + wave * (STAGE_ROWS * EPITCH);
+    r.epi[0] = stage + (lane & 31) * EPITCH + 4 * ESZ * (lane >> 5);        // write: row lane % 32, columns 4 (lane / 32) ..
+    r.epi[1] = stage + (lane / LPR) * EPITCH + (lane % LPR) * 16;           // read: row lane / LPR, chunk lane % LPR
+    // the lane's columns: all valid -> one 16-byte store; some valid (a group boundary inside the chunk)
+    // -> element stores under the mask; none -> nothing
     int mask = 0;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) mask |= (col_t + e >= t.col_lo && col_t + e < t.col_hi) ? (1 << e) : 0;
-    const int off = (row_t * t.ldc + col_t) * 2;
-    r.epi[2] = mask == 0xff ? off : (int)GMM_OOB;
+    for (int e = 0; e < NEL; ++e) mask |= (col_t + e >= t.col_lo && col_t + e < t.col_hi) ? (1 << e) : 0;
+    constexpr int FULL = (1 << NEL) - 1;
+    const int off = (row_t * t.ldc + col_t) * ESZ;
+    r.epi[2] = mask == FULL ? off : (int)GMM_OOB;
     r.epi[3] = t.row_rel0 + row_t;
     r.epi2[0] = off;
-    r.epi2[1] = mask == 0xff ? 0 : mask;
-    partial = ((t.col_lo | t.col_hi) & 7) ? 1 : 0;
-    c_step = 4 * t.ldc * 2;
-  } else {
-    // column c of the wave's block is valid iff (unsigned)(c - col_lo) < col_hi - col_lo
-    const int row_t = wm * WROWS + 4 * (lane >> 5), col_t = wn * 128 + (lane & 31);
-    r.epi[0] = 0;
-    r.epi[1] = col_t - t.col_lo;
-    r.epi[2] = (row_t * t.ldc + col_t) * 4;
-    r.epi[3] = t.row_rel0 + row_t;
-    c_step = t.ldc * 4;
-    n_valid = t.col_hi - t.col_lo;
-    if (n_valid < 0) n_valid = 0;
+    r.epi2[1] = mask == FULL ? 0 : mask;
+    partial = ((t.col_lo | t.col_hi) & (NEL - 1)) ? 1 : 0;
   }
+  const int c_step = (64 / LPR) * t.ldc * ESZ;
+  const int n_valid = 0;
   r.rsrc_a = gmm_make_rsrc(t.a.base, t.a.bytes);
   r.rsrc_b = gmm_make_rsrc(t.b.base, t.b.bytes);
   r.rsrc_c = gmm_make_rsrc(t.c, t.c_bytes);
