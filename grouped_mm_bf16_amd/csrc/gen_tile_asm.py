@@ -530,7 +530,9 @@ def gen_epilogue(v, e, L):
             e("s_waitcnt lgkmcnt(%d)" % min(depth - 1, nrb - 1 - r))
             e("v_cmp_gt_u32 vcc, %s, %s" % (sr(S_ROWCNT), vr(vrow)))
             e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vsel), vr(V_OOB), vr(voff)))
-            e("buffer_store_dwordx4 %s, %s, %s, 0 offen" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
+            # non-temporal: the output is written once and not read by this kernel; kept out of the way, it does
+            # not push operand panels that other workgroups are about to share out of the L2
+            e("buffer_store_dwordx4 %s, %s, %s, 0 offen nt" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
             e("s_bitcmp1_b32 %s, 2" % sr(S_T + 18))
             e("s_cbranch_scc0 L_nopart%d_%s" % (nstore, L))
             for el in range(nel):
