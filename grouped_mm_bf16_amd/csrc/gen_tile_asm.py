@@ -106,8 +106,9 @@ def sr(base, n=1):
 class Variant:
     """tm = MFMA block rows per wave: the tile is 64 tm rows (256 / 128 / 64) by 256 columns."""
 
-    def __init__(self, a_tr, b_tr, out_f32, tm=4, f16=0):
-        self.a_tr, self.b_tr, self.out_f32, self.tm, self.f16 = a_tr, b_tr, out_f32, tm, f16
+    def __init__(self, a_tr, b_tr, out_f32, tm=4, f16=0, b_nt=0):
+        """b_nt: B is copied with the non-temporal hint (a B panel that no other tile reads)."""
+        self.a_tr, self.b_tr, self.out_f32, self.tm, self.f16, self.b_nt = a_tr, b_tr, out_f32, tm, f16, b_nt
         self.dt = "f16" if f16 else "bf16"   # element type of A, B and of a 16-bit output
         assert tm in (1, 2, 4) and (tm == 4 or not a_tr)
         self.tn = 4                      # 32-column MFMA blocks per wave (the wave grid is 2 x 2)
@@ -122,7 +123,8 @@ class Variant:
         self.a_stage = TR_STAGE if a_tr else (64 * tm * 128 if self.stages == 3 else KC_STAGE)
         self.b_stage = TR_STAGE if b_tr else KC_STAGE
         self.b_base = self.stages * self.a_stage   # LDS offset of B buffer 0
-        self.name = "%s%s_%s_%s_m%d" % ("t" if a_tr else "k", "t" if b_tr else "k", self.dt, "f32" if out_f32 else self.dt, 64 * tm)
+        self.name = "%s%s_%s_%s_m%d%s" % ("t" if a_tr else "k", "t" if b_tr else "k", self.dt, "f32" if out_f32 else self.dt, 64 * tm,
+                                          "_bnt" if b_nt else "")
 
     def acc(self, i, j):
         return (self.tn * i + j) * 16
@@ -213,7 +215,8 @@ class Variant:
             out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(vn), vr(vt), sr(s_tail, 2)))
             out.append("v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(tmp), vr(V_OOB), sr(s_oob, 2)))
             src = vr(tmp)
-        out.append("buffer_load_dwordx4 %s, %s, %s offen lds" % (src, sr(S_RA if is_a else S_RB, 4), sr(s_ka if is_a else s_kb)))
+        pol = " nt" if (self.b_nt and not is_a) else ""
+        out.append("buffer_load_dwordx4 %s, %s, %s offen%s lds" % (src, sr(S_RA if is_a else S_RB, 4), sr(s_ka if is_a else s_kb), pol))
         return out
 
 
@@ -580,13 +583,15 @@ def main():
     out.append("#define GMM_TILE_STAGING_BYTES %d" % STAGE_BYTES)
     out.append("#define GMM_TILE_STAGES_SHORT %d" % STAGES_SHORT)
     for f16 in (0, 1):
-        for a_tr, b_tr, f32, tm in [(a, b, f, t) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1)]:
+        for a_tr, b_tr, f32, tm, b_nt in [(a, b, f, t, n) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1) for n in (0, 1)]:
             if tm != 4 and a_tr:
                 continue
-            v = Variant(a_tr, b_tr, f32, tm, f16)
+            if b_nt and tm == 4:
+                continue      # only remainder tiles can be the sole reader of a B panel often enough to matter
+            v = Variant(a_tr, b_tr, f32, tm, f16, b_nt)
             e = gen_variant(v)
             out.append("")
-            out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm, f16))
+            out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm, f16, b_nt))
             out.append("  asm volatile(")
             out.append(e.text())
             out.append("      :")

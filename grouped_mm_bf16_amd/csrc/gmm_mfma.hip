@@ -357,9 +357,13 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       if constexpr (A_TR) {
         gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16>(dsc, lds_base, lane_j, wave);
       } else {
+        // a short tile that holds all rows of its group is the only reader of its B panel
+        const bool sole = m_hi - m_lo <= rows;
         if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16>(dsc, lds_base, lane_j, wave);
-        else if (rows == 128) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2, F16>(dsc, lds_base, lane_j, wave);
-        else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1, F16>(dsc, lds_base, lane_j, wave);
+        else if (rows == 128 && !sole) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2, F16, 0>(dsc, lds_base, lane_j, wave);
+        else if (rows == 128) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2, F16, 1>(dsc, lds_base, lane_j, wave);
+        else if (!sole) gmm_tile_compute<A_TR, B_TR, OUT_F32, 1, F16, 0>(dsc, lds_base, lane_j, wave);
+        else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1, F16, 1>(dsc, lds_base, lane_j, wave);
       }
     }
     if (left <= BATCH) break;

@@ -25,7 +25,9 @@ struct GmmTileRegs {
 
 // TM = MFMA block rows per wave: the tile is 64 * TM rows (256, 128 or 64) by 256 columns.
 // F16 = 1: A, B and a 16-bit output are fp16 instead of bf16 (same layouts, other MFMA and conversion).
-template <int A_TR, int B_TR, int OUT_F32, int TM, int F16>
+// B_NT = 1 (128- and 64-row tiles): B is copied with the non-temporal hint, for a tile that is the only
+// reader of its B panel (it then does not push panels that other tiles share out of the L2).
+template <int A_TR, int B_TR, int OUT_F32, int TM, int F16, int B_NT>
 __device__ __forceinline__ void gmm_tile_asm(GmmTileRegs& r);
 
 #include "gmm_tile_asm.inc"
@@ -130,7 +132,7 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int
   }
 }
 
-template <int A_TR, int B_TR, int OUT_F32, int TM = 4, int F16 = 0>
+template <int A_TR, int B_TR, int OUT_F32, int TM = 4, int F16 = 0, int B_NT = 0>
 __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave) {
   static_assert(TM == 4 || !A_TR, "short tiles exist for a K-contiguous A only");
   constexpr int WROWS = 32 * TM;  // rows of the tile per wave row
@@ -214,5 +216,5 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   const int sc[8] = {nk, a_step, b_step, (int)lds_base, t.row_cnt, c_step, n_valid, wave | (flags << 8)};
 #pragma unroll
   for (int i = 0; i < 8; ++i) r.scal[i] = __builtin_amdgcn_readfirstlane(sc[i]);
-  gmm_tile_asm<A_TR, B_TR, OUT_F32, TM, F16>(r);
+  gmm_tile_asm<A_TR, B_TR, OUT_F32, TM, F16, B_NT>(r);
 }
