@@ -331,8 +331,10 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       // Extents end at the last element of the operand's last row, not at a whole leading dimension: a
       // padded view (ld larger than the row) may end exactly there.
       if (!A_TR) {
+        // rows past the group's last row (jagged rows) are not fetched at all: they read as zeros
+        const int a_rows_end = p.jag == GMM_JAG_M ? m_hi : p.M;
         dsc.a.base = a + int64_t(m0) * lda + k_begin;
-        dsc.a.bytes = (int64_t(p.M - 1 - m0) * lda + (p.K - k_begin)) * 2;
+        dsc.a.bytes = (int64_t(a_rows_end - 1 - m0) * lda + (p.K - k_begin)) * 2;
       } else {
         dsc.a.base = a + int64_t(k_begin) * lda + m0;
         dsc.a.bytes = (int64_t(p.K - 1 - k_begin) * lda + (p.M - m0)) * 2;
