@@ -12,7 +12,7 @@ import threading
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libgrouped_mm_hip.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # enum gmm_path / gmm_dtype / gmm_status of the header
 PATH_AUTO, PATH_GENERIC, PATH_MFMA = 0, 1, 2
@@ -26,9 +26,14 @@ SIGNATURES = {
     "gmm_abi_version": (ctypes.c_int, []),
     "gmm_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "gmm_2d3d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),
+    "gmm_2d3d_gather": (ctypes.c_int, [_vp] * 5 + [_i32] + [_i64] * 4 + [_i64] * 7 + [_i32, _i32, _vp]),
     "gmm_3d3d": (ctypes.c_int, [_vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 9 + [_i32, _i32, _vp]),
     "gmm_2d2d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),
     "gmm_3d2d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),
+    "gmm_moe_route_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "gmm_moe_route": (ctypes.c_int, [_vp, _i64, _i32, _i64, _i64, _i64, _i32] + [_vp] * 5 + [_vp, _i64, _vp]),
+    "gmm_moe_activation": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _vp]),
+    "gmm_moe_combine": (ctypes.c_int, [_vp] * 4 + [_i64] * 6 + [_i32, _vp]),
     "gmm_set_path": (ctypes.c_int, [ctypes.c_int]),
     "gmm_last_path": (ctypes.c_int, []),
     "gmm_set_mfma_config": (ctypes.c_int, [ctypes.c_int]),

@@ -103,9 +103,14 @@ int run(Problem& pr, hipStream_t stream) {
   int align = 1;
   const int forced = g_forced_path.load(std::memory_order_relaxed);
   const bool aligned = mfma_eligible(pr, lay, align);
-  const bool can_asm = aligned && asm_tile_eligible(pr, lay);
+  bool can_asm = aligned && asm_tile_eligible(pr, lay);
+  if (p.gather) {
+    // the assembly tile gathers rows of a K-contiguous first operand whose byte offsets fit 31 bits; the
+    // register-staged MFMA kernel has no gather: everything else goes to the generic family
+    if (can_asm && !(lay.a_kc && int64_t(p.a_rows) * p.a_sm * 2 < (int64_t(1) << 31))) can_asm = false;
+  }
   // fp16 has the assembly tile only (configuration 1); bf16 also the register-staged kernel
-  const bool can_mfma = aligned && (pr.in_dtype == GMM_DT_BF16 || can_asm);
+  const bool can_mfma = aligned && (p.gather ? can_asm : (pr.in_dtype == GMM_DT_BF16 || can_asm));
   if (forced == GMM_PATH_MFMA && !can_mfma) return GMM_ERR_UNSUPPORTED;
   const bool use_mfma = can_mfma && forced != GMM_PATH_GENERIC;
 
@@ -116,6 +121,7 @@ int run(Problem& pr, hipStream_t stream) {
     int cfg = g_forced_config.load(std::memory_order_relaxed);
     if (cfg == GMM_CFG_ASM_256x256 && !can_asm) return GMM_ERR_UNSUPPORTED;
     if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = can_asm ? GMM_CFG_ASM_256x256 : GMM_CFG_REG_256x256;
+    if (p.gather && cfg != GMM_CFG_ASM_256x256) return GMM_ERR_UNSUPPORTED;
     if (pr.in_dtype != GMM_DT_BF16 && cfg != GMM_CFG_ASM_256x256) return GMM_ERR_UNSUPPORTED;
     // the assembly tile stores 16-byte chunks: its tile columns start at multiples of 8 elements
     if (cfg == GMM_CFG_ASM_256x256 && p.jag == GMM_JAG_N) p.align = 8;
@@ -158,6 +164,7 @@ const char* gmm_status_string(int status) {
     case GMM_ERR_BAD_ARGUMENT: return "bad argument (null pointer, size out of range or more than 1023 groups)";
     case GMM_ERR_UNSUPPORTED: return "unsupported dtype combination or forced kernel family not applicable";
     case GMM_ERR_LAUNCH: return "HIP launch failed";
+    case GMM_ERR_WORKSPACE: return "workspace too small for this problem";
     default: return "unknown status";
   }
 }
@@ -169,6 +176,22 @@ int gmm_2d3d(const void* a, const void* b, void* out, const int32_t* offs, int32
   Problem pr{};
   pr.p = GmmParams{a, b, out, offs, G, GMM_JAG_M, int32_t(M_total), int32_t(N), int32_t(K), 1,
                    0, a_sm, a_sk, b_sg, b_sk, b_sn, 0, o_sm, o_sn, 0, 0};
+  pr.in_dtype = in_dtype;
+  pr.out_dtype = out_dtype;
+  return run(pr, static_cast<hipStream_t>(stream));
+}
+
+int gmm_2d3d_gather(const void* a, const int32_t* row_index, const void* b, void* out, const int32_t* offs, int32_t G,
+                    int64_t a_rows, int64_t M_total, int64_t N, int64_t K, int64_t a_sm, int64_t a_sk, int64_t b_sg,
+                    int64_t b_sk, int64_t b_sn, int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype,
+                    void* stream) {
+  if (!dims_ok(M_total, N, K) || !fits_i32(a_rows)) return GMM_ERR_BAD_ARGUMENT;
+  if (!row_index && M_total > 0 && G > 0 && N > 0) return GMM_ERR_BAD_ARGUMENT;
+  Problem pr{};
+  pr.p = GmmParams{a, b, out, offs, G, GMM_JAG_M, int32_t(M_total), int32_t(N), int32_t(K), 1,
+                   0, a_sm, a_sk, b_sg, b_sk, b_sn, 0, o_sm, o_sn, 0, 0};
+  pr.p.gather = row_index;
+  pr.p.a_rows = int32_t(a_rows);
   pr.in_dtype = in_dtype;
   pr.out_dtype = out_dtype;
   return run(pr, static_cast<hipStream_t>(stream));

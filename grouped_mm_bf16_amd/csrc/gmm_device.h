@@ -150,6 +150,12 @@ __device__ __forceinline__ GmmTile gmm_locate_tile2(const GmmParams& p, const in
   return gmm_make_tile2(p, g, lo, hi, cls, local, bn);
 }
 
+// Source row of product row m under a row gather; -1 if the index is outside the source matrix.
+__device__ __forceinline__ int gmm_gather_row(const GmmParams& p, int m) {
+  const int s = p.gather[m];
+  return (s >= 0 && s < p.a_rows) ? s : -1;
+}
+
 // ---- element types -------------------------------------------------------- //
 struct gmm_bf16 { uint16_t bits; };
 struct gmm_f16 { _Float16 v; };

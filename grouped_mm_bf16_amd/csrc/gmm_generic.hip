@@ -48,7 +48,10 @@ __global__ void __launch_bounds__(GNT) gmm_generic_kernel(const GmmParams p) {
           const int r = e / GK, kk = e % GK;
           const int m = tile.m0 + r, k = k0 + kk;
           float v = 0.f;
-          if (m < p.M && k < tile.k_hi) v = gmm_to_float(a[int64_t(m) * p.a_sm + int64_t(k) * p.a_sk]);
+          if (m < p.M && k < tile.k_hi) {
+            const int ms = p.gather ? gmm_gather_row(p, m) : m;   // a row index out of range reads as zeros
+            if (ms >= 0) v = gmm_to_float(a[int64_t(ms) * p.a_sm + int64_t(k) * p.a_sk]);
+          }
           sa[kk][r] = v;
         }
         {
@@ -137,7 +140,9 @@ __global__ void __launch_bounds__(GNT) gmm_wide_kernel(const GmmParams p) {
         int r, kk;
         gmm_wide_coord(tid + i * GNT, a_kc, r, kk);
         const int m = tile.m0 + r, k = k0 + kk;
-        ra[i] = (m < p.M && k < tile.k_hi) ? gmm_to_float(a[int64_t(m) * p.a_sm + int64_t(k) * p.a_sk]) : 0.f;
+        int ms = m < p.M ? m : -1;
+        if (p.gather && ms >= 0) ms = gmm_gather_row(p, m);
+        ra[i] = (ms >= 0 && k < tile.k_hi) ? gmm_to_float(a[int64_t(ms) * p.a_sm + int64_t(k) * p.a_sk]) : 0.f;
         gmm_wide_coord(tid + i * GNT, b_kc, r, kk);
         const int n = tile.n0 + r;
         const int kb = k0 + kk;

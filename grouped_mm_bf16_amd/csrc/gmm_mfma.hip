@@ -330,7 +330,14 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       dsc.b.ld = ldb;
       // Extents end at the last element of the operand's last row, not at a whole leading dimension: a
       // padded view (ld larger than the row) may end exactly there.
-      if (!A_TR) {
+      if (!A_TR && p.gather) {
+        // row gather: the tile's rows come from rows gather[m0 ..] of the whole source matrix
+        dsc.a.base = a + k_begin;
+        dsc.a.bytes = (int64_t(p.a_rows - 1) * lda + (p.K - k_begin)) * 2;
+        dsc.a.gather = p.gather + m0;
+        dsc.a.gather_n = m_hi - m0;
+        dsc.a.src_rows = p.a_rows;
+      } else if (!A_TR) {
         // rows past the group's last row (jagged rows) are not fetched at all: they read as zeros
         const int a_rows_end = p.jag == GMM_JAG_M ? m_hi : p.M;
         dsc.a.base = a + int64_t(m0) * lda + k_begin;

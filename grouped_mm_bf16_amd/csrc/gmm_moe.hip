@@ -1,0 +1,355 @@
+// The mixture-of-experts step either side of the grouped product (declared in include/grouped_mm_hip.h):
+//   routing   top-k experts per token, their softmax weights, and a stable counting sort of the
+//             (token, choice) slots by expert that yields `offs` for the grouped product without the
+//             host ever seeing a count (the reference's benchmark does this with bincount / cumsum and an
+//             offs[-1].item() round trip, bench/bench_2d3d.py:124-139);
+//   activation   SiLU or SwiGLU between the up and the down projection;
+//   combine   out[t] = sum_j weight[t, j] * y[row of slot (t, j)], the un-permute, without atomics.
+// All of it is HBM- or latency-bound integer / elementwise work: coalesced 16-byte accesses, LDS for the
+// histograms and ranks, no matrix cores.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "../../include/grouped_mm_hip.h"
+
+namespace {
+
+constexpr int kMaxExperts = 1023;        // the grouped product takes fewer than 1024 groups
+constexpr int kMaxTopK = 32;
+constexpr int kMaxSortBlocks = 256;      // workgroups of the counting sort (rows of the histogram table)
+constexpr int kSlotsPerSortBlock = 1024; // aimed-at slots per workgroup
+
+
+// ---------------------------------------------------------------- element types
+struct Bf16 { uint16_t bits; };
+struct F16 { _Float16 v; };
+
+__device__ __forceinline__ float to_float(Bf16 x) { return __uint_as_float(uint32_t(x.bits) << 16); }
+__device__ __forceinline__ float to_float(F16 x) { return float(x.v); }
+__device__ __forceinline__ float to_float(float x) { return x; }
+
+template <typename T> __device__ __forceinline__ T from_float(float f);
+template <> __device__ __forceinline__ Bf16 from_float<Bf16>(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return Bf16{uint16_t((u >> 16) | 0x40)};   // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);                                                 // round to nearest even
+  return Bf16{uint16_t(u >> 16)};
+}
+template <> __device__ __forceinline__ F16 from_float<F16>(float f) { return F16{_Float16(f)}; }
+
+template <typename T> struct alignas(16) Vec8 { T v[8]; };
+
+// ---------------------------------------------------------------- wave helpers (64 lanes)
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+  return x;
+}
+__device__ __forceinline__ uint64_t wave_max(uint64_t x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint32_t lo = __shfl_xor(uint32_t(x), o), hi = __shfl_xor(uint32_t(x >> 32), o);
+    const uint64_t y = (uint64_t(hi) << 32) | lo;
+    x = y > x ? y : x;
+  }
+  return x;
+}
+
+// fp32 -> uint32 whose unsigned order is the numeric order (NaN with a clear sign bit sorts above +inf)
+__device__ __forceinline__ uint32_t order_key(float v) {
+  const uint32_t u = __float_as_uint(v + 0.0f);   // -0 becomes +0: the two compare equal
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// ---------------------------------------------------------------- routing 1/4: top-k and weights
+// One wave per token.  Choice j of token t is slot t * k + j.  Ties go to the lower expert index (a stable
+// descending sort).  weight = softmax over the chosen k logits (renorm) or over all E logits.
+template <typename T>
+__global__ void __launch_bounds__(256) moe_topk_kernel(const T* __restrict__ logits, int64_t ld, int tokens, int E, int k,
+                                                       int renorm, int32_t* __restrict__ slot_expert,
+                                                       float* __restrict__ slot_weight) {
+  __shared__ uint32_t keys[4][1024];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= tokens) return;
+  const T* row = logits + int64_t(t) * ld;
+  uint32_t* kw = keys[wave];   // lane l reads and writes entries l, l + 64, ... only
+  for (int e = lane; e < E; e += 64) kw[e] = order_key(to_float(row[e]));
+  uint32_t taken = 0, my_key = 0, top_key = 0;
+  int my_e = 0;
+  for (int j = 0; j < k; ++j) {
+    uint64_t best = 0;
+    for (int e = lane, i = 0; e < E; e += 64, ++i) {
+      const uint64_t c = (uint64_t(kw[e]) << 32) | uint32_t(0xffffffffu - uint32_t(e));
+      if (!((taken >> i) & 1u) && c > best) best = c;
+    }
+    best = wave_max(best);
+    const int e_win = int(0xffffffffu - uint32_t(best));
+    const uint32_t key_win = uint32_t(best >> 32);
+    if ((e_win & 63) == lane) taken |= 1u << (e_win >> 6);
+    if (lane == j) { my_e = e_win; my_key = key_win; }
+    if (j == 0) top_key = key_win;
+  }
+  const float m = key_value(top_key);
+  const float p = lane < k ? __expf(key_value(my_key) - m) : 0.0f;
+  float den;
+  if (renorm) {
+    den = wave_sum(p);
+  } else {
+    float s = 0.0f;
+    for (int e = lane; e < E; e += 64) s += __expf(key_value(kw[e]) - m);
+    den = wave_sum(s);
+  }
+  if (lane < k) {
+    slot_expert[int64_t(t) * k + lane] = my_e;
+    slot_weight[int64_t(t) * k + lane] = p / den;
+  }
+}
+
+// ---------------------------------------------------------------- routing 2/4: per-workgroup histograms
+// Workgroup b counts the experts of slots [b * spb, (b + 1) * spb) into row b of the table.
+__global__ void __launch_bounds__(256) moe_hist_kernel(const int32_t* __restrict__ slot_expert, int slots, int spb, int E,
+                                                       int32_t* __restrict__ table) {
+  __shared__ int32_t hist[1024];
+  for (int e = threadIdx.x; e < E; e += 256) hist[e] = 0;
+  __syncthreads();
+  const int s0 = blockIdx.x * spb, s1 = min(slots, s0 + spb);
+  for (int s = s0 + threadIdx.x; s < s1; s += 256) atomicAdd(&hist[slot_expert[s]], 1);
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) table[int64_t(blockIdx.x) * E + e] = hist[e];
+}
+
+// ---------------------------------------------------------------- routing 3/4: column scan + offs
+// One workgroup of 1024 threads, thread e owns expert e: the table's column e becomes its exclusive prefix
+// over the workgroups, and offs[e] the inclusive prefix of the expert totals.
+__global__ void __launch_bounds__(1024) moe_scan_kernel(int32_t* __restrict__ table, int nb, int E, int32_t* __restrict__ offs) {
+  __shared__ int32_t part[16];
+  const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
+  int run = 0;
+  if (e < E) {
+    for (int b = 0; b < nb; ++b) {
+      const int c = table[int64_t(b) * E + e];
+      table[int64_t(b) * E + e] = run;
+      run += c;
+    }
+  }
+  int incl = run;   // inclusive scan of `run` over the 1024 threads
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int up = __shfl_up(incl, o);
+    if (lane >= o) incl += up;
+  }
+  if (lane == 63) part[wave] = incl;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < wave; ++w) base += part[w];
+  if (e < E) offs[e] = base + incl;
+}
+
+// ---------------------------------------------------------------- routing 4/4: stable scatter
+// Workgroup b places its slots, in slot order, behind what earlier workgroups hold of the same expert:
+// row = offs[e - 1] + (slots of expert e in earlier workgroups) + (earlier slots of e in this workgroup).
+__global__ void __launch_bounds__(256) moe_scatter_kernel(const int32_t* __restrict__ slot_expert, int slots, int spb, int E,
+                                                          int k, const int32_t* __restrict__ table,
+                                                          const int32_t* __restrict__ offs, int32_t* __restrict__ row_token,
+                                                          int32_t* __restrict__ token_rows) {
+  __shared__ int32_t cursor[1024];
+  __shared__ __attribute__((aligned(16))) int32_t chunk[256];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += 256) cursor[e] = table[int64_t(blockIdx.x) * E + e] + (e ? offs[e - 1] : 0);
+  const int s0 = blockIdx.x * spb, s1 = min(slots, s0 + spb);
+  for (int c = s0; c < s1; c += 256) {
+    const int s = c + tid;
+    const int e = s < s1 ? slot_expert[s] : -1;
+    __syncthreads();   // cursor initialised / updated, chunk free
+    chunk[tid] = e;
+    __syncthreads();
+    int before = 0, total = 0;
+    for (int j = 0; j < 256; j += 4) {
+      const int4 q = *reinterpret_cast<const int4*>(&chunk[j]);
+      const int m0 = q.x == e, m1 = q.y == e, m2 = q.z == e, m3 = q.w == e;
+      total += m0 + m1 + m2 + m3;
+      before += (m0 & (j < tid)) + (m1 & (j + 1 < tid)) + (m2 & (j + 2 < tid)) + (m3 & (j + 3 < tid));
+    }
+    int row = 0;
+    if (e >= 0) row = cursor[e] + before;
+    __syncthreads();   // every cursor read done
+    if (e >= 0) {
+      if (before == total - 1) cursor[e] += total;
+      row_token[row] = s / k;
+      token_rows[s] = row;
+    }
+  }
+}
+
+// ---------------------------------------------------------------- activation
+// kind 0: out = silu(h);  kind 1: out = silu(h[:, :inner]) * h[:, inner:2 * inner].  fp32 arithmetic, one
+// rounding.  Each thread handles 8 adjacent elements (16 bytes).
+template <typename T>
+__global__ void __launch_bounds__(256) moe_act_kernel(const T* __restrict__ h, T* __restrict__ out, int64_t rows, int64_t inner,
+                                                      int64_t ld_h, int64_t ld_out, int kind) {
+  const int64_t vec_per_row = inner >> 3, total = rows * vec_per_row;
+  for (int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x; i < total; i += int64_t(gridDim.x) * 256) {
+    const int64_t r = i / vec_per_row, c = (i - r * vec_per_row) << 3;
+    const Vec8<T> g = *reinterpret_cast<const Vec8<T>*>(h + r * ld_h + c);
+    Vec8<T> u, o;
+    if (kind) u = *reinterpret_cast<const Vec8<T>*>(h + r * ld_h + inner + c);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float x = to_float(g.v[j]);
+      float y = x / (1.0f + __expf(-x));
+      if (kind) y *= to_float(u.v[j]);
+      o.v[j] = from_float<T>(y);
+    }
+    *reinterpret_cast<Vec8<T>*>(out + r * ld_out + c) = o;
+  }
+}
+
+// ---------------------------------------------------------------- combine
+// out[t, :] = sum over j < k of slot_weight[t * k + j] * y[token_rows[t * k + j], :], summed in fp32 in the
+// order of j and rounded once.  One workgroup per token; a slot whose row is outside [0, y_rows) adds nothing.
+template <typename T>
+__global__ void __launch_bounds__(256) moe_combine_kernel(const T* __restrict__ y, const int32_t* __restrict__ token_rows,
+                                                          const float* __restrict__ slot_weight, T* __restrict__ out, int k,
+                                                          int64_t H, int64_t y_rows, int64_t ld_y, int64_t ld_out) {
+  __shared__ int32_t rows[kMaxTopK];
+  __shared__ float wts[kMaxTopK];
+  const int64_t t = blockIdx.x;
+  if (threadIdx.x < k) {
+    rows[threadIdx.x] = token_rows[t * k + threadIdx.x];
+    wts[threadIdx.x] = slot_weight[t * k + threadIdx.x];
+  }
+  __syncthreads();
+  for (int64_t c = int64_t(threadIdx.x) << 3; c < H; c += 256 * 8) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int j = 0; j < k; ++j) {
+      const int64_t r = rows[j];
+      if (r < 0 || r >= y_rows) continue;
+      const Vec8<T> v = *reinterpret_cast<const Vec8<T>*>(y + r * ld_y + c);
+      const float w = wts[j];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += w * to_float(v.v[i]);
+    }
+    Vec8<T> o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o.v[i] = from_float<T>(acc[i]);
+    *reinterpret_cast<Vec8<T>*>(out + t * ld_out + c) = o;
+  }
+}
+
+// ---------------------------------------------------------------- host side
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+struct SortPlan {
+  int slots, nb, spb;
+};
+
+bool plan_sort(int64_t tokens, int64_t top_k, SortPlan& pl) {
+  const int64_t slots = tokens * top_k;
+  if (slots < 0 || slots >= (int64_t(1) << 31)) return false;
+  int64_t nb = (slots + kSlotsPerSortBlock - 1) / kSlotsPerSortBlock;
+  if (nb < 1) nb = 1;
+  if (nb > kMaxSortBlocks) nb = kMaxSortBlocks;
+  const int64_t spb = slots ? (slots + nb - 1) / nb : 1;
+  pl.slots = int(slots);
+  pl.spb = int(spb);
+  pl.nb = slots ? int((slots + spb - 1) / spb) : 0;
+  return true;
+}
+
+int route_checked(const void* logits, int64_t ld, int dtype, int64_t tokens, int64_t E, int64_t top_k, int renorm,
+                  int32_t* offs, int32_t* slot_expert, float* slot_weight, int32_t* row_token, int32_t* token_rows,
+                  int32_t* table, size_t table_bytes, hipStream_t stream) {
+  if (tokens < 0 || E < 1 || E > kMaxExperts || top_k < 1 || top_k > kMaxTopK || top_k > E) return GMM_ERR_BAD_ARGUMENT;
+  if (dtype < GMM_DT_BF16 || dtype > GMM_DT_F32) return GMM_ERR_UNSUPPORTED;
+  SortPlan pl;
+  if (!plan_sort(tokens, top_k, pl)) return GMM_ERR_BAD_ARGUMENT;
+  if (!offs) return GMM_ERR_BAD_ARGUMENT;
+  if (tokens > 0 && (!logits || !slot_expert || !slot_weight || !row_token || !token_rows || ld < E)) return GMM_ERR_BAD_ARGUMENT;
+  if (size_t(pl.nb) * size_t(E) * sizeof(int32_t) > table_bytes) return GMM_ERR_WORKSPACE;
+  if (pl.nb > 0 && !table) return GMM_ERR_BAD_ARGUMENT;
+  if (tokens > 0) {
+    const dim3 grid(unsigned((tokens + 3) / 4)), block(256);
+    if (dtype == GMM_DT_BF16)
+      hipLaunchKernelGGL(moe_topk_kernel<Bf16>, grid, block, 0, stream, static_cast<const Bf16*>(logits), ld, int(tokens), int(E),
+                         int(top_k), renorm, slot_expert, slot_weight);
+    else if (dtype == GMM_DT_F16)
+      hipLaunchKernelGGL(moe_topk_kernel<F16>, grid, block, 0, stream, static_cast<const F16*>(logits), ld, int(tokens), int(E),
+                         int(top_k), renorm, slot_expert, slot_weight);
+    else
+      hipLaunchKernelGGL(moe_topk_kernel<float>, grid, block, 0, stream, static_cast<const float*>(logits), ld, int(tokens), int(E),
+                         int(top_k), renorm, slot_expert, slot_weight);
+    hipLaunchKernelGGL(moe_hist_kernel, dim3(pl.nb), dim3(256), 0, stream, slot_expert, pl.slots, pl.spb, int(E), table);
+  }
+  hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, stream, table, pl.nb, int(E), offs);
+  if (tokens > 0)
+    hipLaunchKernelGGL(moe_scatter_kernel, dim3(pl.nb), dim3(256), 0, stream, slot_expert, pl.slots, pl.spb, int(E), int(top_k),
+                       table, offs, row_token, token_rows);
+  return hipGetLastError() == hipSuccess ? GMM_OK : GMM_ERR_LAUNCH;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t gmm_moe_route_workspace_bytes(int64_t tokens, int64_t experts, int64_t top_k) {
+  SortPlan pl;
+  if (tokens < 0 || experts < 1 || experts > kMaxExperts || top_k < 1 || !plan_sort(tokens, top_k, pl)) return -1;
+  return int64_t(pl.nb) * experts * int64_t(sizeof(int32_t));
+}
+
+int gmm_moe_route(const void* logits, int64_t logits_stride, int32_t logits_dtype, int64_t tokens, int64_t experts,
+                  int64_t top_k, int32_t renormalize, int32_t* offs, int32_t* slot_expert, float* slot_weight,
+                  int32_t* row_token, int32_t* token_rows, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (workspace_bytes < 0) return GMM_ERR_BAD_ARGUMENT;
+  return route_checked(logits, logits_stride, logits_dtype, tokens, experts, top_k, renormalize, offs, slot_expert,
+                       slot_weight, row_token, token_rows, static_cast<int32_t*>(workspace), size_t(workspace_bytes),
+                       static_cast<hipStream_t>(stream));
+}
+
+int gmm_moe_activation(const void* h, void* out, int64_t rows, int64_t inner, int64_t h_stride, int64_t out_stride,
+                       int32_t kind, int32_t dtype, void* stream) {
+  if (rows < 0 || inner < 0 || kind < 0 || kind > 1) return GMM_ERR_BAD_ARGUMENT;
+  if (dtype != GMM_DT_BF16 && dtype != GMM_DT_F16) return GMM_ERR_UNSUPPORTED;
+  if (rows == 0 || inner == 0) return GMM_OK;
+  if (!h || !out || (inner & 7) || (h_stride & 7) || (out_stride & 7) || !aligned16(h) || !aligned16(out)) return GMM_ERR_BAD_ARGUMENT;
+  if (h_stride < (kind ? 2 : 1) * inner || out_stride < inner) return GMM_ERR_BAD_ARGUMENT;
+  const int64_t vecs = rows * (inner >> 3);
+  int64_t blocks = (vecs + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  const dim3 grid{unsigned(blocks)}, block{256};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == GMM_DT_BF16)
+    hipLaunchKernelGGL(moe_act_kernel<Bf16>, grid, block, 0, s, static_cast<const Bf16*>(h), static_cast<Bf16*>(out), rows, inner,
+                       h_stride, out_stride, kind);
+  else
+    hipLaunchKernelGGL(moe_act_kernel<F16>, grid, block, 0, s, static_cast<const F16*>(h), static_cast<F16*>(out), rows, inner,
+                       h_stride, out_stride, kind);
+  return hipGetLastError() == hipSuccess ? GMM_OK : GMM_ERR_LAUNCH;
+}
+
+int gmm_moe_combine(const void* y, const int32_t* token_rows, const float* slot_weight, void* out, int64_t tokens,
+                    int64_t top_k, int64_t hidden, int64_t y_rows, int64_t y_stride, int64_t out_stride, int32_t dtype,
+                    void* stream) {
+  if (tokens < 0 || tokens >= (int64_t(1) << 31) || top_k < 1 || top_k > kMaxTopK || hidden < 0 || y_rows < 0) return GMM_ERR_BAD_ARGUMENT;
+  if (dtype != GMM_DT_BF16 && dtype != GMM_DT_F16) return GMM_ERR_UNSUPPORTED;
+  if (tokens == 0 || hidden == 0) return GMM_OK;
+  if (!out || !token_rows || !slot_weight || (y_rows > 0 && !y)) return GMM_ERR_BAD_ARGUMENT;
+  if ((hidden & 7) || (y_stride & 7) || (out_stride & 7) || !aligned16(y) || !aligned16(out)) return GMM_ERR_BAD_ARGUMENT;
+  if (y_stride < hidden || out_stride < hidden) return GMM_ERR_BAD_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid{unsigned(tokens)}, block{256};
+  if (dtype == GMM_DT_BF16)
+    hipLaunchKernelGGL(moe_combine_kernel<Bf16>, grid, block, 0, s, static_cast<const Bf16*>(y), token_rows, slot_weight,
+                       static_cast<Bf16*>(out), int(top_k), hidden, y_rows, y_stride, out_stride);
+  else
+    hipLaunchKernelGGL(moe_combine_kernel<F16>, grid, block, 0, s, static_cast<const F16*>(y), token_rows, slot_weight,
+                       static_cast<F16*>(out), int(top_k), hidden, y_rows, y_stride, out_stride);
+  return hipGetLastError() == hipSuccess ? GMM_OK : GMM_ERR_LAUNCH;
+}
+
+}  // extern "C"

@@ -45,6 +45,10 @@ struct GmmParams {
   int32_t num_wg;     // persistent grid size
   int32_t tall;       // tile list with several heights: rows of a "tall" tile (256 or 128) ...
   int32_t shrt;       // ... and of the shortest tile for group remainders (64), or 0: tall tiles only
+  // Row gather for the first operand (jagged rows only): row r of the product reads row gather[r] of `a`
+  // (which then has `a_rows` rows); null: row r reads row r.
+  const int32_t* gather;
+  int32_t a_rows;
 };
 
 GMM_HD int gmm_cdiv(int a, int b) { return (a + b - 1) / b; }

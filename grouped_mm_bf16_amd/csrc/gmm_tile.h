@@ -77,6 +77,11 @@ struct GmmOperand {
   const uint16_t* base;
   int ld;
   long long bytes;
+  // Row gather (first operand, contiguous along K only): tile row r reads row gather[r] of the matrix at
+  // `base` (which then points at row 0), for r < gather_n; other rows, and indices outside [0, src_rows),
+  // read as zeros.  Null: tile row r is row r from `base`.
+  const int32_t* gather = nullptr;
+  int gather_n = 0, src_rows = 0;
 };
 
 // Description of one tile for the assembly.  klen = number of k elements from k_begin that count.
@@ -96,8 +101,9 @@ struct GmmTileDesc {
 // klen, khead and nk are the same for all lanes: whether the first / last K tile is a whole one is a
 // scalar branch, and only partial ones pay for the per-lane selects.
 template <int TR, int NI>
-__device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int klen, int khead, int nk,
+__device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, const GmmOperand& op, int klen, int khead, int nk,
                                                  gmm_v8i& head, gmm_v8i& full, gmm_v8i& tail) {
+  const int ld = op.ld;
   int kk[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -106,7 +112,12 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, int ld, int
       const int row = wave * (NI * 8) + i * 8 + (lane >> 3);
       const int c = (lane & 7) ^ gmm_swz(row);
       kk[i] = c * 8;
-      full[i] = row * ld * 2 + c * 16;
+      int src = row;
+      if (op.gather) {
+        src = row < op.gather_n ? op.gather[row] : -1;
+        if (src >= op.src_rows) src = -1;
+      }
+      full[i] = src >= 0 ? src * ld * 2 + c * 16 : (int)GMM_OOB;
     } else {
       const int blk = wave * 8 + i;
       kk[i] = 8 * (blk >> 2) + (blk & 3) + 4 * (lane >> 5);
@@ -140,8 +151,8 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   const int wm = wave & 1, wn = wave >> 1;
   const int nk = (t.klen + GMM_TILE_K - 1) / GMM_TILE_K;
   GmmTileRegs r;
-  gmm_copy_offsets<A_TR, 2 * TM>(lane, wave, t.a.ld, t.klen, t.khead, nk, r.voa_head, r.voa, r.voa_tail);
-  gmm_copy_offsets<B_TR, 8>(lane, wave, t.b.ld, t.klen, t.khead, nk, r.vob_head, r.vob, r.vob_tail);
+  gmm_copy_offsets<A_TR, 2 * TM>(lane, wave, t.a, t.klen, t.khead, nk, r.voa_head, r.voa, r.voa_tail);
+  gmm_copy_offsets<B_TR, 8>(lane, wave, t.b, t.klen, t.khead, nk, r.vob_head, r.vob, r.vob_tail);
   const int q = lane >> 4, ii = lane & 15;
 #pragma unroll
   for (int s = 0; s < 4; ++s) {

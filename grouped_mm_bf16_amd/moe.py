@@ -1,0 +1,179 @@
+"""The mixture-of-experts step around the grouped product, entirely on the device:
+
+    routing (top-k, weights, stable sort by expert -> offs)  ->  up projection with the token gather done
+    by the tile's own copies  ->  SiLU / SwiGLU  ->  down projection  ->  weighted un-permute.
+
+The reference ships the grouped product only; its benchmark prepares rows that are already sorted by expert
+and gets ``offs`` from ``bincount(...).cumsum(0)`` with a host round trip (``bench/bench_2d3d.py:124-149``).
+Here no count ever reaches the host: the kernels read ``offs`` from device memory, and every buffer is sized
+by ``tokens * top_k``, which the host knows.
+
+Forward only (inference); the functions take and return plain tensors.
+"""
+from __future__ import annotations
+
+import contextlib
+from typing import NamedTuple
+
+import torch
+
+from . import _lib
+from .kernels import _dtype_code, _require_gpu, grouped_mm_2d3d
+
+ACTIVATIONS = {"silu": 0, "swiglu": 1}
+
+
+class Routing(NamedTuple):
+    """What :func:`moe_route` returns; S = tokens * top_k slots, slot t * top_k + j is choice j of token t."""
+    offs: torch.Tensor          # int32 [E]  end offset of each expert's rows (what grouped_mm takes)
+    slot_expert: torch.Tensor   # int32 [S]  expert of each slot
+    slot_weight: torch.Tensor   # float32 [S] combine weight of each slot
+    row_token: torch.Tensor     # int32 [S]  token whose activations row r of the sorted matrix holds
+    token_rows: torch.Tensor    # int32 [S]  row of each slot (inverse permutation)
+
+
+def _guard(t: torch.Tensor):
+    return torch.cuda.device(t.device) if t.device.index != torch.cuda.current_device() else contextlib.nullcontext()
+
+
+def moe_route(router_logits: torch.Tensor, top_k: int, renormalize: bool = True) -> Routing:
+    """Top-k routing and the stable sort of the slots by expert.
+
+    router_logits [T, E] (bf16, fp16 or fp32, last dimension contiguous).  Ties go to the lower expert index;
+    weights are the softmax over the chosen logits (``renormalize``) or the chosen entries of the softmax
+    over all experts.
+    """
+    _require_gpu(router_logits)
+    if router_logits.dim() != 2:
+        raise RuntimeError("router_logits has to be 2D [tokens, experts]")
+    if router_logits.size(0) and router_logits.stride(1) != 1:
+        raise RuntimeError("router_logits must be contiguous along the experts")
+    T, E = router_logits.shape
+    if not 1 <= top_k <= min(E, 32):
+        raise RuntimeError(f"top_k must be in [1, min(experts, 32)], got {top_k} for {E} experts")
+    if E > 1023:
+        raise RuntimeError("Can't process more than 1024 groups")
+    lib = _lib.load()
+    dev, S = router_logits.device, T * top_k
+    i32 = dict(device=dev, dtype=torch.int32)
+    r = Routing(torch.empty(E, **i32), torch.empty(S, **i32), torch.empty(S, device=dev, dtype=torch.float32),
+                torch.empty(S, **i32), torch.empty(S, **i32))
+    ws_bytes = lib.gmm_moe_route_workspace_bytes(T, E, top_k)
+    if ws_bytes < 0:
+        raise RuntimeError("moe_route: sizes out of range")
+    ws = torch.empty(max(ws_bytes, 4) // 4, **i32)
+    with _guard(router_logits):
+        rc = lib.gmm_moe_route(router_logits.data_ptr(), router_logits.stride(0) if T else E,
+                               _dtype_code(router_logits.dtype), T, E, top_k, int(bool(renormalize)),
+                               r.offs.data_ptr(), r.slot_expert.data_ptr(), r.slot_weight.data_ptr(),
+                               r.row_token.data_ptr(), r.token_rows.data_ptr(), ws.data_ptr(), ws_bytes,
+                               torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "moe_route")
+    return r
+
+
+def grouped_mm_gathered(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tensor, offs: torch.Tensor,
+                        out: torch.Tensor | None = None) -> torch.Tensor:
+    """``grouped_mm(a[row_index], b, offs=offs)`` without materialising ``a[row_index]``.
+
+    a [R_src, K], row_index int32 [M_total], b [G, K, N], offs int32 [G]; returns [M_total, N] in a's dtype.
+    An index outside [0, R_src) reads a row of zeros.
+    """
+    _require_gpu(a, row_index, b, offs)
+    if a.dim() != 2 or b.dim() != 3:
+        raise RuntimeError("grouped_mm_gathered takes a 2D first and a 3D second operand")
+    if a.dtype != b.dtype:
+        raise RuntimeError("mat_a and mat_b must have the same dtype")
+    if a.size(1) != b.size(1):
+        raise RuntimeError("contraction dimension of mat_a and mat_b must match")
+    if row_index.dtype != torch.int32 or row_index.dim() != 1 or not row_index.is_contiguous():
+        raise RuntimeError("row_index has to be a contiguous 1D int32 tensor")
+    if offs.dtype != torch.int32 or offs.dim() != 1:
+        raise RuntimeError("Offsets have to be int32")
+    if offs.numel() != b.size(0):
+        raise RuntimeError("matrix batch sizes have to match")
+    M, N = row_index.numel(), b.size(2)
+    if out is None:
+        out = torch.empty(M, N, device=a.device, dtype=a.dtype)
+    if M == 0 or N == 0:
+        return out
+    if a.size(1) == 0:
+        return out.zero_()
+    lib = _lib.load()
+    with _guard(a):
+        rc = lib.gmm_2d3d_gather(a.data_ptr(), row_index.data_ptr(), b.data_ptr(), out.data_ptr(), offs.data_ptr(),
+                                 offs.numel(), a.size(0), M, N, a.size(1), a.stride(0), a.stride(1),
+                                 b.stride(0), b.stride(1), b.stride(2), out.stride(0), out.stride(1),
+                                 _dtype_code(a.dtype), _dtype_code(out.dtype), torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "grouped_mm_gathered launch")
+    return out
+
+
+def moe_activation(h: torch.Tensor, kind: str = "swiglu", out: torch.Tensor | None = None) -> torch.Tensor:
+    """``silu(h)`` or, for "swiglu", ``silu(h[:, :I]) * h[:, I:]`` with I = h.size(1) // 2 (fp32 arithmetic,
+    one rounding).  h [R, I or 2I], bf16 or fp16, row-major."""
+    _require_gpu(h)
+    if kind not in ACTIVATIONS:
+        raise RuntimeError(f"unknown activation {kind!r}; have {sorted(ACTIVATIONS)}")
+    code = ACTIVATIONS[kind]
+    if h.dim() != 2 or (h.numel() and h.stride(1) != 1):
+        raise RuntimeError("moe_activation takes a row-major 2D tensor")
+    if code and h.size(1) % 2:
+        raise RuntimeError("swiglu needs an even number of columns")
+    inner = h.size(1) // 2 if code else h.size(1)
+    if out is None:
+        out = torch.empty(h.size(0), inner, device=h.device, dtype=h.dtype)
+    lib = _lib.load()
+    with _guard(h):
+        rc = lib.gmm_moe_activation(h.data_ptr(), out.data_ptr(), h.size(0), inner, h.stride(0) if h.size(0) else inner,
+                                    out.stride(0) if h.size(0) else inner, code, _dtype_code(h.dtype),
+                                    torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "moe_activation")
+    return out
+
+
+def moe_combine(y: torch.Tensor, routing: Routing, tokens: int, top_k: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = sum_j slot_weight[t, j] * y[token_rows[t, j]] in fp32, rounded once.  y [S, H] row-major."""
+    _require_gpu(y)
+    if y.dim() != 2 or (y.numel() and y.stride(1) != 1):
+        raise RuntimeError("moe_combine takes a row-major 2D tensor")
+    H = y.size(1)
+    if out is None:
+        out = torch.empty(tokens, H, device=y.device, dtype=y.dtype)
+    lib = _lib.load()
+    with _guard(y):
+        rc = lib.gmm_moe_combine(y.data_ptr(), routing.token_rows.data_ptr(), routing.slot_weight.data_ptr(), out.data_ptr(),
+                                 tokens, top_k, H, y.size(0), y.stride(0) if y.size(0) else H, out.stride(0) if tokens else H,
+                                 _dtype_code(y.dtype), torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "moe_combine")
+    return out
+
+
+def moe_forward(x: torch.Tensor, router_logits: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, top_k: int,
+                activation: str = "swiglu", renormalize: bool = True) -> torch.Tensor:
+    """One mixture-of-experts feed-forward layer.
+
+    x [T, H]; router_logits [T, E]; w_up [E, H, I] ("silu") or [E, H, 2I] ("swiglu": gate columns first, then
+    up columns); w_down [E, I, H].  Returns [T, H] in x's dtype:
+    ``sum_j weight[t, j] * (act(x[t] @ w_up[e_tj]) @ w_down[e_tj])``.
+    Intermediate results are rounded to x's dtype after each of the three stages, as separate layers would.
+    """
+    if x.dim() != 2 or router_logits.dim() != 2 or x.size(0) != router_logits.size(0):
+        raise RuntimeError("x [T, H] and router_logits [T, E] must agree on T")
+    if w_up.dim() != 3 or w_down.dim() != 3 or w_up.size(0) != router_logits.size(1) or w_down.size(0) != w_up.size(0):
+        raise RuntimeError("w_up [E, H, I or 2I] and w_down [E, I, H] must agree with router_logits on E")
+    if activation not in ACTIVATIONS:
+        raise RuntimeError(f"unknown activation {activation!r}; have {sorted(ACTIVATIONS)}")
+    inner = w_up.size(2) // 2 if ACTIVATIONS[activation] else w_up.size(2)
+    if w_up.size(1) != x.size(1) or w_down.size(1) != inner or w_down.size(2) != x.size(1):
+        raise RuntimeError("weight shapes do not chain: x [T, H], w_up [E, H, I or 2I], w_down [E, I, H]")
+    T = x.size(0)
+    routing = moe_route(router_logits, top_k, renormalize)
+    h = grouped_mm_gathered(x, routing.row_token, w_up, routing.offs)
+    act = moe_activation(h, activation)
+    del h
+    y = torch.empty(act.size(0), w_down.size(2), device=x.device, dtype=x.dtype)
+    grouped_mm_2d3d(act, w_down, routing.offs, y)   # rows are already sorted by expert
+    del act
+    return moe_combine(y, routing, T, top_k)
+

@@ -28,13 +28,14 @@
 extern "C" {
 #endif
 
-#define GMM_ABI_VERSION 1
+#define GMM_ABI_VERSION 2
 
 enum gmm_status {
   GMM_OK = 0,
   GMM_ERR_BAD_ARGUMENT = 1, /* null pointer, negative size, G out of range, bad stride */
   GMM_ERR_UNSUPPORTED = 2,  /* dtype combination or forced path not available */
-  GMM_ERR_LAUNCH = 3        /* the HIP runtime refused the launch */
+  GMM_ERR_LAUNCH = 3,       /* the HIP runtime refused the launch */
+  GMM_ERR_WORKSPACE = 4     /* the workspace passed in is smaller than the problem needs */
 };
 
 enum gmm_dtype { GMM_DT_BF16 = 0, GMM_DT_F16 = 1, GMM_DT_F32 = 2 };
@@ -55,6 +56,21 @@ int gmm_2d3d(const void* a, const void* b, void* out, const int32_t* offs, int32
              int64_t b_stride_g, int64_t b_stride_k, int64_t b_stride_n,
              int64_t out_stride_m, int64_t out_stride_n,
              int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/* 2D x 3D with the rows of the first operand gathered on the fly:
+ *   out[r, :] = a[row_index[r], :] @ b[g(r)]   for r < offs[G-1], g(r) the group that owns row r.
+ * a [a_rows, K], row_index int32[M_total] (device), b [G, K, N], out [M_total, N].  An index outside
+ * [0, a_rows) reads a row of zeros.  This is gmm_2d3d applied to a[row_index] without materialising the
+ * permuted copy: the token gather that a mixture-of-experts layer performs between routing and the up
+ * projection (the reference's benchmark starts from rows already sorted, bench/bench_2d3d.py:140-149).
+ * The assembly tile takes it when `a` is contiguous along K and a_rows * a_stride_m * 2 < 2^31. */
+int gmm_2d3d_gather(const void* a, const int32_t* row_index, const void* b, void* out,
+                    const int32_t* offs, int32_t G, int64_t a_rows,
+                    int64_t M_total, int64_t N, int64_t K,
+                    int64_t a_stride_m, int64_t a_stride_k,
+                    int64_t b_stride_g, int64_t b_stride_k, int64_t b_stride_n,
+                    int64_t out_stride_m, int64_t out_stride_n,
+                    int32_t in_dtype, int32_t out_dtype, void* stream);
 
 /* 3D x 3D: out[g] = a[g] @ b[g]
  * a [G, M, K], b [G, K, N], out [G, M, N].
@@ -85,6 +101,43 @@ int gmm_3d2d(const void* a, const void* b, void* out, const int32_t* offs, int32
              int64_t b_stride_k, int64_t b_stride_n,
              int64_t out_stride_m, int64_t out_stride_n,
              int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/* ---- The mixture-of-experts step either side of the grouped product.  The reference has no such code;
+ * its benchmark builds the sorted rows and `offs` with torch on the host side (bench/bench_2d3d.py:124-149:
+ * randint / bincount / cumsum and an offs[-1].item() round trip).  Here everything stays on the device.
+ *
+ * Routing.  For each of `tokens` rows of `logits` [tokens, experts] (row stride logits_stride elements,
+ * dtype a gmm_dtype) pick the top_k largest (ties: lower expert index first; logits must not be NaN), in
+ * descending order.  Choice j of token t is SLOT t * top_k + j.  Outputs (device memory):
+ *   slot_expert int32[tokens * top_k]   expert of each slot
+ *   slot_weight float[tokens * top_k]   softmax over the token's chosen logits (renormalize != 0), or the
+ *                                       chosen entries of the softmax over all experts (renormalize == 0)
+ *   offs        int32[experts]          end offsets of the experts' row ranges (inclusive prefix of counts)
+ *   row_token   int32[tokens * top_k]   rows sorted by expert, stably in slot order: the token of each row
+ *   token_rows  int32[tokens * top_k]   the row of each slot (inverse of the sort)
+ * experts <= 1023, top_k <= min(experts, 32), tokens * top_k < 2^31.  `workspace` is device memory of at
+ * least gmm_moe_route_workspace_bytes(...) bytes (per-workgroup expert histograms; contents need not be
+ * initialised); too small a workspace returns GMM_ERR_WORKSPACE.  Four launches on `stream`, no host sync. */
+int64_t gmm_moe_route_workspace_bytes(int64_t tokens, int64_t experts, int64_t top_k);
+int gmm_moe_route(const void* logits, int64_t logits_stride, int32_t logits_dtype,
+                  int64_t tokens, int64_t experts, int64_t top_k, int32_t renormalize,
+                  int32_t* offs, int32_t* slot_expert, float* slot_weight,
+                  int32_t* row_token, int32_t* token_rows,
+                  void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Activation between the two projections, bf16 or fp16, fp32 arithmetic and one rounding:
+ *   kind 0: out[r, c] = silu(h[r, c]);   kind 1 (SwiGLU): out[r, c] = silu(h[r, c]) * h[r, inner + c],
+ * for r < rows, c < inner.  inner and both strides multiples of 8 elements, 16-byte aligned bases. */
+int gmm_moe_activation(const void* h, void* out, int64_t rows, int64_t inner,
+                       int64_t h_stride, int64_t out_stride, int32_t kind, int32_t dtype, void* stream);
+
+/* Un-permute and weighted sum: out[t, :] = sum_{j < top_k} slot_weight[t * top_k + j] * y[token_rows[t * top_k + j], :],
+ * added in fp32 in the order of j and rounded once (no atomics: the result does not depend on timing).
+ * y [y_rows, hidden], out [tokens, hidden], bf16 or fp16; hidden and strides multiples of 8, 16-byte aligned
+ * bases.  A slot whose row is outside [0, y_rows) contributes nothing. */
+int gmm_moe_combine(const void* y, const int32_t* token_rows, const float* slot_weight, void* out,
+                    int64_t tokens, int64_t top_k, int64_t hidden, int64_t y_rows,
+                    int64_t y_stride, int64_t out_stride, int32_t dtype, void* stream);
 
 /* Test and tuning hooks (the reference exposes its tile knobs through environment
  * variables read in the launcher, kernels.py:590-634; tests force tiles through

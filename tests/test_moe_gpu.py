@@ -1,0 +1,278 @@
+"""The mixture-of-experts step on a real MI355X, through the C ABI, against oracle/moe_oracle.py:
+routing bit for bit (integers) and to fp32 rounding (weights); the gathered product against the grouped
+oracle on the permuted rows; activation and combine to one rounding of the output type; the whole layer at
+small, Mixtral and fine-grained sizes."""
+import pytest
+import torch
+
+from grouped_mm_bf16_amd import kernels as K_
+from grouped_mm_bf16_amd import moe
+from oracle import grouped_mm_oracle as oracle
+from oracle import moe_oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def rnd(gen, *shape, dtype=torch.bfloat16, scale=1.0):
+    return (torch.randn(*shape, generator=gen) * scale).to(dtype)
+
+
+def offs_of(sizes):
+    return torch.tensor(sizes, dtype=torch.int64).cumsum(0).to(torch.int32)
+
+
+def check_routing(got: moe.Routing, want: moe_oracle.Routing):
+    torch.cuda.synchronize()
+    assert torch.equal(got.slot_expert.cpu(), want.slot_expert), "chosen experts differ"
+    assert torch.equal(got.offs.cpu(), want.offs), "offs differ"
+    assert torch.equal(got.row_token.cpu(), want.row_token), "row order differs"
+    assert torch.equal(got.token_rows.cpu(), want.token_rows), "slot -> row map differs"
+    torch.testing.assert_close(got.slot_weight.cpu(), want.slot_weight, rtol=2e-5, atol=1e-7)
+
+
+# ------------------------------------------------------------------ routing
+@pytest.mark.parametrize("T,E,k", [(1, 1, 1), (7, 8, 2), (64, 8, 8), (1000, 128, 8), (4096, 128, 8), (8192, 8, 2),
+                                   (700, 1023, 32), (3, 70, 1), (300000, 3, 1), (32768, 64, 8)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_routing_matches_the_oracle(T, E, k, dtype):
+    """bf16 logits tie often: the lower expert index must win, as in a stable descending sort."""
+    gen = torch.Generator().manual_seed(T + E + k)
+    logits = torch.randn(T, E, generator=gen).to(dtype)
+    for renorm in (True, False):
+        got = moe.moe_route(logits.to(DEV), k, renormalize=renorm)
+        check_routing(got, moe_oracle.route(logits, k, renorm))
+
+
+def test_routing_fp16_skewed_padded_and_empty():
+    gen = torch.Generator().manual_seed(3)
+    # skew: most tokens pick expert 0, several experts stay empty
+    logits = torch.randn(2048, 32, generator=gen)
+    logits[:, 0] += 4.0
+    logits[:, 20:] -= 30.0
+    lh = logits.half()
+    check_routing(moe.moe_route(lh.to(DEV), 2), moe_oracle.route(lh, 2))
+    want = moe_oracle.route(lh, 2)
+    assert (want.offs[20:] == want.offs[19]).all()
+    # a view with a row stride wider than E
+    wide = torch.full((2048, 40), float("inf"), device=DEV, dtype=torch.float16)
+    wide[:, :32] = lh.to(DEV)
+    check_routing(moe.moe_route(wide[:, :32], 2), want)
+    # no tokens: offs is all zero, nothing else is written
+    r = moe.moe_route(torch.empty(0, 8, device=DEV), 2)
+    torch.cuda.synchronize()
+    assert r.offs.tolist() == [0] * 8 and r.slot_expert.numel() == 0
+
+
+def test_routing_rejects_what_it_cannot_do():
+    lg = torch.zeros(4, 8, device=DEV)
+    with pytest.raises(RuntimeError):
+        moe.moe_route(lg, 9)
+    with pytest.raises(RuntimeError):
+        moe.moe_route(lg, 0)
+    with pytest.raises(RuntimeError):
+        moe.moe_route(torch.zeros(4, 1024, device=DEV), 2)
+    with pytest.raises(RuntimeError):
+        moe.moe_route(lg.t(), 2)
+    from grouped_mm_bf16_amd import _lib
+    lib = _lib.load()
+    need = lib.gmm_moe_route_workspace_bytes(5000, 128, 8)
+    assert need == 40 * 128 * 4
+    r = [torch.empty(40000, device=DEV, dtype=torch.int32) for _ in range(5)]
+    rc = lib.gmm_moe_route(torch.zeros(5000, 128, device=DEV).data_ptr(), 128, _lib.DT_F32, 5000, 128, 8, 1,
+                           r[0].data_ptr(), r[1].data_ptr(), r[2].view(torch.float32).data_ptr(), r[3].data_ptr(),
+                           r[4].data_ptr(), r[0].data_ptr(), need - 4, None)
+    assert rc == 4 and b"workspace" in lib.gmm_status_string(rc)
+
+
+# ------------------------------------------------------------------ gathered product
+SIZES = [77, 0, 1, 130, 64, 200, 15, 16, 17, 31, 33, 300]
+
+
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("dtype,K,N,path", [(torch.bfloat16, 136, 264, "mfma"), (torch.float16, 136, 264, "mfma"),
+                                            (torch.bfloat16, 4096, 512, "mfma"), (torch.bfloat16, 33, 29, "generic"),
+                                            (torch.float32, 40, 24, "generic"), (torch.bfloat16, 136, 264, "generic")])
+def test_gathered_product_equals_the_product_of_the_gathered_rows(dtype, K, N, path, b_col):
+    gen = torch.Generator().manual_seed(K + N)
+    G, M, S = len(SIZES), sum(SIZES), 401
+    a = rnd(gen, S, K, dtype=dtype)
+    b = rnd(gen, G, K, N, dtype=dtype, scale=0.1)
+    idx = torch.randint(0, S, (M + 9,), generator=gen).to(torch.int32)   # repeats; 9 rows past offs[-1]
+    idx[5], idx[300] = -1, S                                            # outside the source: rows of zeros
+    offs = offs_of(SIZES)
+    bd = b.to(DEV)
+    if b_col:
+        bd = bd.transpose(1, 2).contiguous().transpose(1, 2)
+    out = torch.full((M + 9, N), float("nan"), device=DEV, dtype=dtype)
+    with K_.forced_path(path):
+        moe.grouped_mm_gathered(a.to(DEV), idx.to(DEV), bd, offs.to(DEV), out=out)
+        torch.cuda.synchronize()
+        assert K_.last_path() == path
+        # the same kernel on a materialised copy: bit-identical
+        az = torch.cat([a, torch.zeros(1, K, dtype=dtype)])
+        src = idx.long().clone()
+        src[(src < 0) | (src >= S)] = S
+        plain = torch.full_like(out, float("nan"))
+        K_.grouped_mm_2d3d(az[src].to(DEV), bd, offs.to(DEV), plain)
+        torch.cuda.synchronize()
+    got = out.cpu()
+    assert torch.isnan(got[M:].float()).all(), "rows past offs[-1] were written"
+    assert torch.equal(got[:M].view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       plain.cpu()[:M].view(torch.int16 if dtype != torch.float32 else torch.int32))
+    want = oracle.grouped_mm(az[src], b, offs)
+    if dtype == torch.float32:
+        torch.testing.assert_close(got[:M], want[:M], rtol=3e-4, atol=3e-4)
+    else:
+        oracle.assert_close(got[:M], want[:M], K)
+    assert (got[5] == 0).all() and (got[300] == 0).all()
+
+
+def test_gathered_product_on_views_and_large_sources():
+    """Source rows 24 elements apart from their extent, at a storage offset; a source whose byte offsets need
+    all 31 bits still takes the assembly tile, a larger one goes to the generic family."""
+    gen = torch.Generator().manual_seed(77)
+    K, N, S = 136, 264, 90
+    a = rnd(gen, S, K)
+    buf = torch.full((16 + S * (K + 24) - 24,), float("nan"), device=DEV, dtype=torch.bfloat16)
+    av = torch.as_strided(buf, (S, K), (K + 24, 1), 16)
+    av.copy_(a)
+    sizes = [40, 0, 3, 100]
+    idx = torch.randint(0, S, (sum(sizes),), generator=gen).to(torch.int32)
+    b = rnd(gen, len(sizes), K, N, scale=0.1)
+    with K_.forced_path("mfma"):
+        got = moe.grouped_mm_gathered(av, idx.to(DEV), b.to(DEV), offs_of(sizes).to(DEV))
+        torch.cuda.synchronize()
+    oracle.assert_close(got.cpu(), oracle.grouped_mm(a[idx.long()], b, offs_of(sizes)), K)
+    # 2^31 bytes of source: rows * ld * 2 == 2^31 exactly is refused by the tile, taken by the generic kernels
+    S2, K2 = 1 << 17, 8192
+    big = torch.zeros(S2, K2, device=DEV, dtype=torch.bfloat16)
+    big[S2 - 1] = 1.0
+    idx2 = torch.tensor([S2 - 1, 0, S2 - 1], dtype=torch.int32, device=DEV)
+    b2 = torch.ones(1, K2, 8, device=DEV, dtype=torch.bfloat16)
+    got = moe.grouped_mm_gathered(big, idx2, b2, torch.tensor([3], dtype=torch.int32, device=DEV))
+    torch.cuda.synchronize()
+    assert K_.last_path() == "generic"
+    assert got.float().cpu().tolist() == [[8192.0] * 8, [0.0] * 8, [8192.0] * 8]
+    got = moe.grouped_mm_gathered(big[: S2 - 8], idx2 - 8, b2, torch.tensor([3], dtype=torch.int32, device=DEV))
+    torch.cuda.synchronize()
+    assert K_.last_path() == "mfma"
+    assert got.float().cpu().tolist() == [[0.0] * 8, [0.0] * 8, [0.0] * 8]
+    idx3 = torch.tensor([S2 - 9, S2 - 1, 0], dtype=torch.int32, device=DEV)   # last valid row; out of range; first
+    big[S2 - 9] = 2.0
+    got = moe.grouped_mm_gathered(big[: S2 - 8], idx3, b2, torch.tensor([3], dtype=torch.int32, device=DEV))
+    torch.cuda.synchronize()
+    assert got.float().cpu().tolist() == [[16384.0] * 8, [0.0] * 8, [0.0] * 8]
+
+
+# ------------------------------------------------------------------ activation, combine
+def ulp_close(got, want, dtype):
+    """Equal up to one unit in the last place of the 16-bit type (fast exp and fused multiply-adds on the device)."""
+    eps = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    torch.testing.assert_close(got.float(), want.float(), rtol=eps, atol=1e-6 if dtype == torch.bfloat16 else 1e-7)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("kind", ["silu", "swiglu"])
+def test_activation(kind, dtype):
+    gen = torch.Generator().manual_seed(21)
+    h = rnd(gen, 333, 272, dtype=dtype, scale=3.0)
+    h[0, :8] = torch.tensor([0.0, -0.0, 80.0, -80.0, float("inf"), 1e-3, -1e-3, 11.0]).to(dtype)
+    got = moe.moe_activation(h.to(DEV), kind).cpu()
+    want = moe_oracle.activation(h, kind)
+    assert got.shape == want.shape
+    ok = torch.isfinite(want.float())
+    ulp_close(got[ok], want[ok], dtype)
+    # a view: rows of a wider matrix
+    wide = torch.full((333, 304), float("nan"), device=DEV, dtype=dtype)
+    wide[:, :272] = h.to(DEV)
+    got2 = moe.moe_activation(wide[:, :272], kind).cpu()
+    assert torch.equal(got2.view(torch.int16), got.view(torch.int16))
+    assert moe.moe_activation(torch.empty(0, 16, device=DEV, dtype=dtype), kind).shape == (0, 8 if kind == "swiglu" else 16)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,k,H", [(1, 1, 8), (50, 2, 264), (300, 8, 2048), (17, 32, 40)])
+def test_combine(T, k, H, dtype):
+    gen = torch.Generator().manual_seed(T + k + H)
+    E = 40
+    r = moe_oracle.route(torch.randn(T, E, generator=gen), k)
+    y = rnd(gen, T * k, H, dtype=dtype)
+    dev_r = moe.Routing(*(t.to(DEV) for t in r))
+    got = moe.moe_combine(y.to(DEV), dev_r, T, k).cpu()
+    ulp_close(got, moe_oracle.combine(y, r, T, k), dtype)
+    # a slot that points outside y adds nothing
+    rows = r.token_rows.clone()
+    rows[0] = T * k
+    rows[-1] = -1
+    r2 = r._replace(token_rows=rows)
+    got = moe.moe_combine(y.to(DEV), moe.Routing(*(t.to(DEV) for t in r2)), T, k).cpu()
+    y0 = torch.cat([y, torch.zeros(1, H, dtype=dtype)])
+    rows0 = rows.clone()
+    rows0[rows0 < 0] = T * k
+    ulp_close(got, moe_oracle.combine(y0, r2._replace(token_rows=rows0), T, k), dtype)
+
+
+# ------------------------------------------------------------------ the whole layer
+def layer_case(seed, T, H, I, E, k, kind, dtype=torch.bfloat16, skew=0.0, wscale=None, on_device=False):
+    """Inputs with unit-size activations at every stage; big cases draw x and the weights on the device (the
+    host generator needs most of a minute for Mixtral's two billion weights) and copy them back for the oracle."""
+    gen = torch.Generator().manual_seed(seed)
+    logits = torch.randn(T, E, generator=gen)
+    if skew:
+        logits += skew * torch.randn(E, generator=gen)
+    n_up = 2 * I if kind == "swiglu" else I
+    s_up, s_down = (wscale, wscale) if wscale else (H ** -0.5, 2 * I ** -0.5)
+    if on_device:
+        dgen = torch.Generator(device=DEV).manual_seed(seed)
+        mk = lambda *shape, scale: (torch.randn(*shape, generator=dgen, device=DEV) * scale).to(dtype).cpu()
+        return mk(T, H, scale=1.0), logits, mk(E, H, n_up, scale=s_up), mk(E, I, H, scale=s_down)
+    return (rnd(gen, T, H, dtype=dtype), logits, rnd(gen, E, H, n_up, dtype=dtype, scale=s_up),
+            rnd(gen, E, I, H, dtype=dtype, scale=s_down))
+
+
+def run_layer(x, logits, w_up, w_down, k, kind, renorm=True):
+    got = moe.moe_forward(x.to(DEV), logits.to(DEV), w_up.to(DEV), w_down.to(DEV), k, kind, renorm)
+    torch.cuda.synchronize()
+    want = moe_oracle.moe_forward(x, logits, w_up, w_down, k, kind, renorm)
+    # three stages, each within the grouped product's bar; the last contraction runs over I
+    oracle.assert_close(got.cpu(), want, w_down.shape[1])
+    # and as a whole far inside one rounding of the 16-bit type (differences come from rounding flips only)
+    rel = float((got.cpu().double() - want.double()).norm() / want.double().norm())
+    assert rel < 4e-3, rel
+    return got
+
+
+@pytest.mark.parametrize("kind", ["silu", "swiglu"])
+@pytest.mark.parametrize("T,H,I,E,k", [(1, 64, 64, 4, 1), (130, 136, 264, 6, 2), (257, 256, 512, 16, 4), (64, 128, 72, 128, 8)])
+def test_layer_small(T, H, I, E, k, kind):
+    case = layer_case(T + E, T, H, I, E, k, kind)
+    run_layer(*case, k, kind)
+    run_layer(*case, k, kind, renorm=False)
+
+
+def test_layer_fp16_and_dense_pin():
+    """fp16; and the device result against the token-by-token fp64 formulation directly."""
+    x, logits, w_up, w_down = layer_case(5, 48, 64, 96, 5, 2, "swiglu", dtype=torch.float16)
+    got = run_layer(x, logits, w_up, w_down, 2, "swiglu")
+    dense = moe_oracle.moe_dense(x, logits, w_up, w_down, 2, "swiglu")
+    torch.testing.assert_close(got.cpu().double(), dense, rtol=2e-2, atol=2e-3)
+
+
+def test_layer_mixtral_size():
+    """8192 tokens, hidden 4096, inner 14336, 8 experts, top 2, SwiGLU: the up projection is the headline
+    workload with the gate and up weights side by side."""
+    x, logits, w_up, w_down = layer_case(0, 8192, 4096, 14336, 8, 2, "swiglu", wscale=0.02, on_device=True)
+    logits[:, 0] += 1.0
+    run_layer(x, logits, w_up, w_down, 2, "swiglu")
+    assert K_.last_path() == "mfma"
+
+
+def test_layer_fine_grained_size():
+    """4096 tokens, hidden 2048, inner 768, 128 experts, top 8, skewed popularity (empty and one-row experts)."""
+    x, logits, w_up, w_down = layer_case(1, 4096, 2048, 768, 128, 8, "swiglu", skew=1.5, wscale=0.02, on_device=True)
+    r = moe_oracle.route(logits, 8)
+    sizes = torch.diff(r.offs, prepend=torch.zeros(1, dtype=torch.int32))
+    assert (sizes == 0).sum() > 10 and (sizes == 1).any() and (sizes < 16).sum() > 40
+    run_layer(x, logits, w_up, w_down, 8, "swiglu")
+    assert K_.last_path() == "mfma"
