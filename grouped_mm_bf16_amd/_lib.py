@@ -32,6 +32,7 @@ SIGNATURES = {
     "gmm_3d2d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),
     "gmm_moe_route_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "gmm_moe_route": (ctypes.c_int, [_vp, _i64, _i32, _i64, _i64, _i64, _i32] + [_vp] * 5 + [_vp, _i64, _vp]),
+    "gmm_moe_route_noalloc": (ctypes.c_int, [_vp, _i64, _i32, _i64, _i64, _i64, _i32] + [_vp] * 5 + [_vp]),
     "gmm_moe_activation": (ctypes.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _vp]),
     "gmm_moe_combine": (ctypes.c_int, [_vp] * 4 + [_i64] * 6 + [_i32, _vp]),
     "gmm_set_path": (ctypes.c_int, [ctypes.c_int]),

@@ -9,6 +9,7 @@
 // histograms and ranks, no matrix cores.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 
 #include "../../include/grouped_mm_hip.h"
@@ -19,7 +20,16 @@ constexpr int kMaxExperts = 1023;        // the grouped product takes fewer than
 constexpr int kMaxTopK = 32;
 constexpr int kMaxSortBlocks = 256;      // workgroups of the counting sort (rows of the histogram table)
 constexpr int kSlotsPerSortBlock = 1024; // aimed-at slots per workgroup
+constexpr int kScratchInts = 64 * 1024;  // built-in histogram table of the entry point that allocates nothing
 
+// Histogram table of gmm_moe_route_noalloc: 256 KiB, one copy per GPU, held until the process ends.  In host
+// code this name is only a handle for hipGetSymbolAddress; the device address it returns for the current
+// device is what the kernels get.  Every entry the kernels read is written earlier in the same call (the
+// histogram kernel fills rows 0 .. nb-1 completely), so nothing needs clearing between calls.
+static __device__ __align__(256) int32_t scratch[kScratchInts];
+
+constexpr int kMaxDevices = 64;
+std::atomic<int32_t*> g_scratch_ptr[kMaxDevices];
 
 // ---------------------------------------------------------------- element types
 struct Bf16 { uint16_t bits; };
@@ -292,6 +302,20 @@ int route_checked(const void* logits, int64_t ld, int dtype, int64_t tokens, int
   return hipGetLastError() == hipSuccess ? GMM_OK : GMM_ERR_LAUNCH;
 }
 
+// Address of the current device's copy of `scratch`, looked up on the first call on that device.
+int32_t* device_scratch() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  int32_t* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) return nullptr;
+    p = static_cast<int32_t*>(sym);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  return p;
+}
+
 }  // namespace
 
 extern "C" {
@@ -308,6 +332,16 @@ int gmm_moe_route(const void* logits, int64_t logits_stride, int32_t logits_dtyp
   if (workspace_bytes < 0) return GMM_ERR_BAD_ARGUMENT;
   return route_checked(logits, logits_stride, logits_dtype, tokens, experts, top_k, renormalize, offs, slot_expert,
                        slot_weight, row_token, token_rows, static_cast<int32_t*>(workspace), size_t(workspace_bytes),
+                       static_cast<hipStream_t>(stream));
+}
+
+int gmm_moe_route_noalloc(const void* logits, int64_t logits_stride, int32_t logits_dtype, int64_t tokens, int64_t experts,
+                          int64_t top_k, int32_t renormalize, int32_t* offs, int32_t* slot_expert, float* slot_weight,
+                          int32_t* row_token, int32_t* token_rows, void* stream) {
+  int32_t* table = device_scratch();
+  if (!table) return GMM_ERR_LAUNCH;
+  return route_checked(logits, logits_stride, logits_dtype, tokens, experts, top_k, renormalize, offs, slot_expert,
+                       slot_weight, row_token, token_rows, table, sizeof(int32_t) * size_t(kScratchInts),
                        static_cast<hipStream_t>(stream));
 }
 

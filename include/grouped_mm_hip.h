@@ -125,6 +125,19 @@ int gmm_moe_route(const void* logits, int64_t logits_stride, int32_t logits_dtyp
                   int32_t* row_token, int32_t* token_rows,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
+/* gmm_moe_route without a workspace argument.  No counterpart in the reference: it is for callers that
+ * cannot allocate device memory or pass a workspace around (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  The histogram table lives in a 256 KiB array that the library
+ * holds on every GPU it runs on until the process ends; the call allocates nothing.  Problems whose
+ * gmm_moe_route_workspace_bytes(...) exceeds 262144 bytes are refused with GMM_ERR_WORKSPACE (any problem
+ * with experts <= 256 fits; with 1023 experts up to 65536 slots).  All calls on one GPU share that array:
+ * calls that may overlap on one GPU (different streams, different threads) race and must be serialised by
+ * the caller.  Outputs and everything else as gmm_moe_route. */
+int gmm_moe_route_noalloc(const void* logits, int64_t logits_stride, int32_t logits_dtype,
+                          int64_t tokens, int64_t experts, int64_t top_k, int32_t renormalize,
+                          int32_t* offs, int32_t* slot_expert, float* slot_weight,
+                          int32_t* row_token, int32_t* token_rows, void* stream);
+
 /* Activation between the two projections, bf16 or fp16, fp32 arithmetic and one rounding:
  *   kind 0: out[r, c] = silu(h[r, c]);   kind 1 (SwiGLU): out[r, c] = silu(h[r, c]) * h[r, inner + c],
  * for r < rows, c < inner.  inner and both strides multiples of 8 elements, 16-byte aligned bases. */
