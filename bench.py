@@ -365,6 +365,51 @@ def run_workload(name, steps, warmup, torch, dev, path="auto", wall=True):
     return w, {"ms_per_step": ms_per_step, "family": family, "roofline": roof, "parity": "ok"}
 
 
+MOE_LAYERS = {   # tokens, hidden, inner, experts, top_k
+    "moe_mixtral": (8192, 4096, 14336, 8, 2),
+    "moe_fine": (4096, 2048, 768, 128, 8),
+}
+
+
+def run_moe(name, steps, warmup, torch, dev):
+    """One mixture-of-experts feed-forward layer (routing, gathered up projection, SwiGLU, down projection,
+    weighted un-permute), all on the device; kernel time of the whole layer from HIP events.  Parity: the
+    first 256 tokens against the oracle (tokens are independent of each other)."""
+    from grouped_mm_bf16_amd import moe
+    from oracle import grouped_mm_oracle as oracle
+    from oracle import moe_oracle
+    T, H, I, E, k = MOE_LAYERS[name]
+    g = torch.Generator(device=dev).manual_seed(7)
+    bf = torch.bfloat16
+    x = torch.randn(T, H, generator=g, device=dev).to(bf)
+    logits = torch.randn(T, E, generator=g, device=dev)
+    if name == "moe_fine":
+        logits += 1.5 * torch.randn(E, generator=g, device=dev)      # skewed popularity: empty and tiny experts
+    else:
+        logits[:, 0] += 1.0
+    w_up = (torch.randn(E, H, 2 * I, generator=g, device=dev) * 0.02).to(bf)
+    w_down = (torch.randn(E, I, H, generator=g, device=dev) * 0.02).to(bf)
+    out = moe.moe_forward(x, logits, w_up, w_down, k)
+    torch.cuda.synchronize()
+    n = 256
+    want = moe_oracle.moe_forward(x[:n].cpu(), logits[:n].cpu(), w_up.cpu(), w_down.cpu(), k)
+    oracle.assert_close(out[:n].cpu(), want, I, what=f"bench parity {name}")
+    for _ in range(warmup):
+        moe.moe_forward(x, logits, w_up, w_down, k)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for e0, e1 in evs:
+        e0.record()
+        moe.moe_forward(x, logits, w_up, w_down, k)
+        e1.record()
+    torch.cuda.synchronize()
+    ms = statistics.mean(e0.elapsed_time(e1) for e0, e1 in evs)
+    flops = 2 * T * k * H * 2 * I + 2 * T * k * I * H
+    return {"workload": f"MoE layer: {T} tokens, hidden {H}, inner {I} (SwiGLU), {E} experts, top {k}, bf16",
+            "ms": round(ms, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 2), "bound": "mfma" if name == "moe_mixtral" else "hbm",
+            "frac": round(flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4) if name == "moe_mixtral" else None,
+            "parity": "ok", "steps": steps}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -372,10 +417,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="mixtral",
                     choices=["mixtral", "readme", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "plain",
-                             "copy", "mfma_only"])
+                             "copy", "mfma_only", "moe_mixtral", "moe_fine"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true",
-                    help="skip the short runs of the other BASELINE configurations (the `configs` object)")
+                    help="skip the short runs of the other benchmark configurations (the `configs` object)")
     ap.add_argument("--library-comparator", action="store_true",
                     help="also time PyTorch-ROCm's own torch.nn.functional.grouped_mm on the same tensors (context only)")
     ap.add_argument("--path", default="auto", choices=["auto", "mfma", "generic"])
@@ -409,6 +454,12 @@ def main():
     if args.workload == "mfma_only":
         mfma_only(args, torch, dev)
         return
+    if args.workload in MOE_LAYERS:
+        rec = run_moe(args.workload, args.steps, args.warmup, torch, dev)
+        print(json.dumps({"metric": "MoE feed-forward layer, useful TFLOP/s of the two projections", "value": rec["tflops"],
+                          "unit": "TFLOP/s", "n_gpus": 1, "warmup": args.warmup, "ms_per_step": rec["ms"],
+                          "higher_is_better": True, "dtype": "bf16", "data": "synthetic", "config": rec}))
+        return
 
     w, r = run_workload(args.workload, args.steps, args.warmup, torch, dev, args.path)
     tflops = w["flops"] / (r["ms_per_step"] * 1e-3) / 1e12
@@ -431,7 +482,7 @@ def main():
         rec["cpu_baseline"] = cpu_baseline(w, torch)
     del w
     if args.workload == "mixtral" and not args.no_configs:
-        # The other BASELINE configurations, a few steps each (kernel time from HIP events; the headline
+        # The other benchmark configurations, a few steps each (kernel time from HIP events; the headline
         # fields above are the Mixtral workload's alone).
         rec["configs"] = {}
         for name in ("readme", "batched", "batched_colmajor", "fine", "kgrouped"):
@@ -446,6 +497,12 @@ def main():
                     "traffic": ri["roofline"]["traffic"], "parity": ri["parity"], "steps": 10}
                 del wi
             except Exception as ex:   # a config that fails must not take the headline down with it
+                rec["configs"][name] = {"parity": "FAILED", "error": repr(ex)[:300]}
+        # the layer around the product (routing, gather, activation, un-permute)
+        for name in MOE_LAYERS:
+            try:
+                rec["configs"][name] = run_moe(name, 10, 3, torch, dev)
+            except Exception as ex:
                 rec["configs"][name] = {"parity": "FAILED", "error": repr(ex)[:300]}
     print(json.dumps(rec))
 

@@ -56,14 +56,24 @@ __device__ __forceinline__ float wave_sum(float x) {
   for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
   return x;
 }
-__device__ __forceinline__ uint64_t wave_max(uint64_t x) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const uint32_t lo = __shfl_xor(uint32_t(x), o), hi = __shfl_xor(uint32_t(x >> 32), o);
-    const uint64_t y = (uint64_t(hi) << 32) | lo;
-    x = y > x ? y : x;
+// Maximum over the wave with data-parallel-primitive moves: prefix maxima inside each row of 16 lanes
+// (row_shr 1, 2, 4, 8), then lane 15 of a row into the next row (row_bcast15 into rows 1 and 3) and lane 31
+// into rows 2 and 3 (row_bcast31); lane 63 ends up with the maximum of all 64.  Lanes a move does not reach
+// take 0, the identity.
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
+#define GMM_DPP_UMAX(ctrl, rows)                                                        \
+  {                                                                                     \
+    const uint32_t t = uint32_t(__builtin_amdgcn_update_dpp(0, int(v), ctrl, rows, 0xf, false)); \
+    v = t > v ? t : v;                                                                  \
   }
-  return x;
+  GMM_DPP_UMAX(0x111, 0xf)
+  GMM_DPP_UMAX(0x112, 0xf)
+  GMM_DPP_UMAX(0x114, 0xf)
+  GMM_DPP_UMAX(0x118, 0xf)
+  GMM_DPP_UMAX(0x142, 0xa)
+  GMM_DPP_UMAX(0x143, 0xc)
+#undef GMM_DPP_UMAX
+  return uint32_t(__builtin_amdgcn_readlane(int(v), 63));
 }
 
 // fp32 -> uint32 whose unsigned order is the numeric order (NaN with a clear sign bit sorts above +inf)
@@ -91,15 +101,22 @@ __global__ void __launch_bounds__(256) moe_topk_kernel(const T* __restrict__ log
   for (int e = lane; e < E; e += 64) kw[e] = order_key(to_float(row[e]));
   uint32_t taken = 0, my_key = 0, top_key = 0;
   int my_e = 0;
+  const int per_lane = (E + 63) >> 6;
   for (int j = 0; j < k; ++j) {
-    uint64_t best = 0;
-    for (int e = lane, i = 0; e < E; e += 64, ++i) {
-      const uint64_t c = (uint64_t(kw[e]) << 32) | uint32_t(0xffffffffu - uint32_t(e));
-      if (!((taken >> i) & 1u) && c > best) best = c;
+    // this lane's best entry that is still free (lowest index among equals), then the wave's best key
+    uint32_t best = 0;
+    int best_i = -1;
+    for (int i = 0; i < per_lane; ++i) {
+      const int e = lane + (i << 6);
+      if (e < E && !((taken >> i) & 1u) && (best_i < 0 || kw[e] > best)) { best = kw[e]; best_i = i; }
     }
-    best = wave_max(best);
-    const int e_win = int(0xffffffffu - uint32_t(best));
-    const uint32_t key_win = uint32_t(best >> 32);
+    const uint32_t key_win = wave_umax(best_i >= 0 ? best : 0u);
+    // lowest expert index among the lanes that hold that key: lowest i first, then lowest lane
+    int e_win = 0;
+    for (int i = 0; i < per_lane; ++i) {
+      const uint64_t holders = __ballot(best_i == i && best == key_win);
+      if (holders) { e_win = (i << 6) + __ffsll((unsigned long long)holders) - 1; break; }
+    }
     if ((e_win & 63) == lane) taken |= 1u << (e_win >> 6);
     if (lane == j) { my_e = e_win; my_key = key_win; }
     if (j == 0) top_key = key_win;
@@ -141,10 +158,16 @@ __global__ void __launch_bounds__(1024) moe_scan_kernel(int32_t* __restrict__ ta
   const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
   int run = 0;
   if (e < E) {
-    for (int b = 0; b < nb; ++b) {
-      const int c = table[int64_t(b) * E + e];
-      table[int64_t(b) * E + e] = run;
-      run += c;
+    // eight independent loads at a time (each costs a trip to L2), then their exclusive prefixes
+    for (int b0 = 0; b0 < nb; b0 += 8) {
+      int c[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) c[i] = b0 + i < nb ? table[int64_t(b0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (b0 + i < nb) table[int64_t(b0 + i) * E + e] = run;
+        run += c[i];
+      }
     }
   }
   int incl = run;   // inclusive scan of `run` over the 1024 threads
@@ -161,37 +184,46 @@ __global__ void __launch_bounds__(1024) moe_scan_kernel(int32_t* __restrict__ ta
 }
 
 // ---------------------------------------------------------------- routing 4/4: stable scatter
-// Workgroup b places its slots, in slot order, behind what earlier workgroups hold of the same expert:
-// row = offs[e - 1] + (slots of expert e in earlier workgroups) + (earlier slots of e in this workgroup).
-__global__ void __launch_bounds__(256) moe_scatter_kernel(const int32_t* __restrict__ slot_expert, int slots, int spb, int E,
-                                                          int k, const int32_t* __restrict__ table,
-                                                          const int32_t* __restrict__ offs, int32_t* __restrict__ row_token,
-                                                          int32_t* __restrict__ token_rows) {
+// Workgroup b (one wave) places its slots, in slot order, behind what earlier workgroups hold of the same
+// expert: row = offs[e - 1] + (slots of expert e in earlier workgroups) + (earlier slots of e in this one).
+// 64 slots at a time: the lanes that hold the same expert find each other with one ballot per bit of the
+// expert index, and a lane's rank among them is the population count of the lower lanes in that set.
+__global__ void __launch_bounds__(64) moe_scatter_kernel(const int32_t* __restrict__ slot_expert, int slots, int spb, int E,
+                                                         int k, const int32_t* __restrict__ table,
+                                                         const int32_t* __restrict__ offs, int32_t* __restrict__ row_token,
+                                                         int32_t* __restrict__ token_rows) {
   __shared__ int32_t cursor[1024];
-  __shared__ __attribute__((aligned(16))) int32_t chunk[256];
-  const int tid = threadIdx.x;
-  for (int e = tid; e < E; e += 256) cursor[e] = table[int64_t(blockIdx.x) * E + e] + (e ? offs[e - 1] : 0);
+  const int lane = threadIdx.x;
+  for (int e = lane; e < E; e += 64) cursor[e] = table[int64_t(blockIdx.x) * E + e] + (e ? offs[e - 1] : 0);
+  __syncthreads();
   const int s0 = blockIdx.x * spb, s1 = min(slots, s0 + spb);
-  for (int c = s0; c < s1; c += 256) {
-    const int s = c + tid;
-    const int e = s < s1 ? slot_expert[s] : -1;
-    __syncthreads();   // cursor initialised / updated, chunk free
-    chunk[tid] = e;
-    __syncthreads();
-    int before = 0, total = 0;
-    for (int j = 0; j < 256; j += 4) {
-      const int4 q = *reinterpret_cast<const int4*>(&chunk[j]);
-      const int m0 = q.x == e, m1 = q.y == e, m2 = q.z == e, m3 = q.w == e;
-      total += m0 + m1 + m2 + m3;
-      before += (m0 & (j < tid)) + (m1 & (j + 1 < tid)) + (m2 & (j + 2 < tid)) + (m3 & (j + 3 < tid));
-    }
-    int row = 0;
-    if (e >= 0) row = cursor[e] + before;
-    __syncthreads();   // every cursor read done
-    if (e >= 0) {
-      if (before == total - 1) cursor[e] += total;
-      row_token[row] = s / k;
-      token_rows[s] = row;
+  const int bits = E > 1 ? 32 - __clz(E - 1) : 0;   // bits that can differ between expert indices
+  const uint64_t lower = (uint64_t(1) << lane) - 1;
+  for (int c4 = s0; c4 < s1; c4 += 256) {
+    int ev[4];   // four chunks' loads in flight at once: each is a trip to L2 or further
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ev[i] = c4 + 64 * i + lane < s1 ? slot_expert[c4 + 64 * i + lane] : -1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int s = c4 + 64 * i + lane, e = ev[i];
+      const bool live = e >= 0;
+      if (c4 + 64 * i >= s1) break;   // uniform
+      uint64_t same = __ballot(live);
+      for (int bit = 0; bit < bits; ++bit) {
+        const bool on = (e >> bit) & 1;
+        const uint64_t with_bit = __ballot(on && live);
+        same &= on ? with_bit : ~with_bit;
+      }
+      const int before = __popcll(same & lower), total = __popcll(same);
+      int row = 0;
+      if (live) row = cursor[e] + before;
+      __syncthreads();   // every lane has read its cursor
+      if (live) {
+        if (before == total - 1) cursor[e] += total;
+        row_token[row] = s / k;
+        token_rows[s] = row;
+      }
+      __syncthreads();
     }
   }
 }
@@ -297,7 +329,7 @@ int route_checked(const void* logits, int64_t ld, int dtype, int64_t tokens, int
   }
   hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, stream, table, pl.nb, int(E), offs);
   if (tokens > 0)
-    hipLaunchKernelGGL(moe_scatter_kernel, dim3(pl.nb), dim3(256), 0, stream, slot_expert, pl.slots, pl.spb, int(E), int(top_k),
+    hipLaunchKernelGGL(moe_scatter_kernel, dim3(pl.nb), dim3(64), 0, stream, slot_expert, pl.slots, pl.spb, int(E), int(top_k),
                        table, offs, row_token, token_rows);
   return hipGetLastError() == hipSuccess ? GMM_OK : GMM_ERR_LAUNCH;
 }

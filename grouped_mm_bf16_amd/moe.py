@@ -55,13 +55,15 @@ def moe_route(router_logits: torch.Tensor, top_k: int, renormalize: bool = True)
         raise RuntimeError("Can't process more than 1024 groups")
     lib = _lib.load()
     dev, S = router_logits.device, T * top_k
-    i32 = dict(device=dev, dtype=torch.int32)
-    r = Routing(torch.empty(E, **i32), torch.empty(S, **i32), torch.empty(S, device=dev, dtype=torch.float32),
-                torch.empty(S, **i32), torch.empty(S, **i32))
     ws_bytes = lib.gmm_moe_route_workspace_bytes(T, E, top_k)
     if ws_bytes < 0:
         raise RuntimeError("moe_route: sizes out of range")
-    ws = torch.empty(max(ws_bytes, 4) // 4, **i32)
+    # one allocation for the five results and the workspace (each allocation costs microseconds of host time)
+    buf = torch.empty(E + 4 * S + ws_bytes // 4, device=dev, dtype=torch.int32)
+    cut = [E, S, S, S, S]
+    parts = torch.split(buf[:E + 4 * S], cut)
+    r = Routing(parts[0], parts[1], parts[2].view(torch.float32), parts[3], parts[4])
+    ws = buf[E + 4 * S:]
     with _guard(router_logits):
         rc = lib.gmm_moe_route(router_logits.data_ptr(), router_logits.stride(0) if T else E,
                                _dtype_code(router_logits.dtype), T, E, top_k, int(bool(renormalize)),
