@@ -487,14 +487,14 @@ def main():
         rec["configs"] = {}
         for name in ("readme", "batched", "batched_colmajor", "fine", "kgrouped"):
             try:
-                wi, ri = run_workload(name, 10, 3, torch, dev, args.path, wall=False)
+                wi, ri = run_workload(name, 30, 10, torch, dev, args.path, wall=False)
                 k_avg = ri["roofline"]["kernel_ms_avg"]
                 rec["configs"][name] = {
                     "workload": wi["desc"], "kernel_family": ri["family"], "ms": k_avg,
                     "tflops": round(wi["flops"] / (k_avg * 1e-3) / 1e12, 2),
                     "gbs": round(wi["bytes"] / (k_avg * 1e-3) / 1e9, 1),
                     "bound": wi["bound"], "frac": ri["roofline"]["frac"] if wi["bound"] != "latency" else None,
-                    "traffic": ri["roofline"]["traffic"], "parity": ri["parity"], "steps": 10}
+                    "traffic": ri["roofline"]["traffic"], "parity": ri["parity"], "steps": 30}
                 del wi
             except Exception as ex:   # a config that fails must not take the headline down with it
                 rec["configs"][name] = {"parity": "FAILED", "error": repr(ex)[:300]}

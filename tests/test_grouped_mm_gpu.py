@@ -146,6 +146,31 @@ def test_2d3d_boundary_lists_mfma(sizes, b_col):
     check(out, a, b, offs_of(sizes), 72, path="mfma")
 
 
+SMALL_GROUPS = [1, 15, 16, 17, 31, 33, 0, 1, 1, 63, 64, 65, 127, 129, 2]
+
+
+@pytest.mark.parametrize("tall,shrt", [(-1, -1), (256, 64), (256, 0), (128, 64), (128, 0)])
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("K,N", [(72, 264), (2048, 768)])
+def test_small_groups_on_every_tile_height(K, N, b_col, tall, shrt):
+    """Groups of 1, 15, 16, 17, 31, 33 ... rows (what a fine-grained expert layer produces): each row is owned
+    by exactly its group whatever heights the tiles have, and rows of neighbouring groups inside one tile's
+    extent are neither read into the product nor written."""
+    gen = torch.Generator().manual_seed(K + N)
+    sizes = SMALL_GROUPS
+    m = sum(sizes)
+    a, b = rnd(gen, m + 5, K), rnd(gen, len(sizes), K, N, scale=0.05)
+    a[m:] = float("nan")                       # rows past offs[-1]: never part of any product
+    bd = b.to(DEV)
+    if b_col:
+        bd = bd.transpose(1, 2).contiguous().transpose(1, 2)
+    out = torch.full((m + 5, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    with K_.forced_tile_heights(tall, shrt):
+        K_.grouped_mm_2d3d(a.to(DEV), bd, offs_of(sizes).to(DEV), out)
+        torch.cuda.synchronize()
+    check(out, a, b, offs_of(sizes), K, path="mfma")
+
+
 def test_rows_past_the_last_offset_are_not_written():
     gen = torch.Generator().manual_seed(5)
     a, b = rnd(gen, 40, 64), rnd(gen, 2, 64, 48)
