@@ -27,6 +27,7 @@ SIGNATURES = {
     "gmm_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "gmm_2d3d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),
     "gmm_2d3d_gather": (ctypes.c_int, [_vp] * 5 + [_i32] + [_i64] * 4 + [_i64] * 7 + [_i32, _i32, _vp]),
+    "gmm_2d3d_swiglu": (ctypes.c_int, [_vp] * 5 + [_i32] + [_i64] * 4 + [_i64] * 7 + [_i32, _vp]),
     "gmm_3d3d": (ctypes.c_int, [_vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 9 + [_i32, _i32, _vp]),
     "gmm_2d2d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),
     "gmm_3d2d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),

@@ -54,6 +54,7 @@ COPY_SCHEDULE = (8, 8, 0, 0)
 
 PITCH = 272           # bytes per staged row of 128 bf16 (256 + 16: shifts banks per row)
 PITCH32 = 528         # ... of 128 fp32 (512 + 16)
+PITCH_ACT = 144       # ... of the 64 gated values a wave's 128 columns give (128 + 16)
 TR_BLOCK = 1088       # two k rows of 512 bytes + 64 bytes pad
 KC_STAGE = 256 * 64 * 2
 TR_STAGE = 32 * TR_BLOCK
@@ -106,9 +107,13 @@ def sr(base, n=1):
 class Variant:
     """tm = MFMA block rows per wave: the tile is 64 tm rows (256 / 128 / 64) by 256 columns."""
 
-    def __init__(self, a_tr, b_tr, out_f32, tm=4, f16=0, b_nt=0):
-        """b_nt: B is copied with the non-temporal hint (a B panel that no other tile reads)."""
+    def __init__(self, a_tr, b_tr, out_f32, tm=4, f16=0, b_nt=0, act=0):
+        """b_nt: B is copied with the non-temporal hint (a B panel that no other tile reads).
+        act: SwiGLU epilogue -- of each 128 columns the first 64 are gates and the last 64 their partners;
+        the tile stores silu(gate) * partner, 128 columns of a 16-bit output per 256 columns of the product."""
         self.a_tr, self.b_tr, self.out_f32, self.tm, self.f16, self.b_nt = a_tr, b_tr, out_f32, tm, f16, b_nt
+        self.act = act
+        assert not (act and (out_f32 or a_tr))
         self.dt = "f16" if f16 else "bf16"   # element type of A, B and of a 16-bit output
         assert tm in (1, 2, 4) and (tm == 4 or not a_tr)
         self.tn = 4                      # 32-column MFMA blocks per wave (the wave grid is 2 x 2)
@@ -123,8 +128,8 @@ class Variant:
         self.a_stage = TR_STAGE if a_tr else (64 * tm * 128 if self.stages == 3 else KC_STAGE)
         self.b_stage = TR_STAGE if b_tr else KC_STAGE
         self.b_base = self.stages * self.a_stage   # LDS offset of B buffer 0
-        self.name = "%s%s_%s_%s_m%d%s" % ("t" if a_tr else "k", "t" if b_tr else "k", self.dt, "f32" if out_f32 else self.dt, 64 * tm,
-                                          "_bnt" if b_nt else "")
+        self.name = "%s%s_%s_%s_m%d%s%s" % ("t" if a_tr else "k", "t" if b_tr else "k", self.dt, "f32" if out_f32 else self.dt, 64 * tm,
+                                            "_bnt" if b_nt else "", "_swiglu" if act else "")
 
     def acc(self, i, j):
         return (self.tn * i + j) * 16
@@ -488,9 +493,10 @@ def gen_epilogue(v, e, L):
     f32 = v.out_f32
     esz = 4 if f32 else 2
     nel = 16 // esz                       # elements of a 16-byte chunk
-    pitch = PITCH32 if f32 else PITCH
+    pitch = PITCH32 if f32 else (PITCH_ACT if v.act else PITCH)
     ipp = 1 if f32 else v.tm              # MFMA block rows per pass
-    rpi = 1024 // (32 * v.tn * esz)       # rows per read-back instruction (64 lanes x 16 bytes)
+    ncol = 64 if v.act else 32 * v.tn     # elements of a staged row
+    rpi = 1024 // (ncol * esz)            # rows per read-back instruction (64 lanes x 16 bytes)
     depth = 4
     regs = [t + 4 * x for x in range(depth)]          # read-back data, 4 registers each
     voff, vrow, vsel = t + 24, t + 25, t + 26
@@ -512,6 +518,35 @@ def gen_epilogue(v, e, L):
         k = 0
         for il in range(min(ipp, v.tm - p0)):
             i = p0 + il
+            if v.act:
+                # silu(g) * u = g * u / (1 + 2^(-g log2 e)); gate block j pairs with block j + 2 (64 columns on).
+                # Four elements advance together, so no result of a transcendental is read by the next instruction.
+                for j in range(2):
+                    for q in range(4):
+                        b = t + 12 * (k % 2)
+                        k += 1
+                        g0, u0 = v.acc(i, j) + 4 * q, v.acc(i, j + 2) + 4 * q
+                        for r in range(4):
+                            e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), g0 + r))
+                        for r in range(4):
+                            e("v_accvgpr_read_b32 %s, a%d" % (vr(b + 4 + r), u0 + r))
+                        for r in range(4):
+                            e("v_mul_f32 %s, 0xbfb8aa3b, %s" % (vr(b + 8 + r), vr(b + r)))
+                        for r in range(4):
+                            e("v_exp_f32 %s, %s" % (vr(b + 8 + r), vr(b + 8 + r)))
+                        e("s_nop 0")
+                        for r in range(4):
+                            e("v_add_f32 %s, 1.0, %s" % (vr(b + 8 + r), vr(b + 8 + r)))
+                        for r in range(4):
+                            e("v_rcp_f32 %s, %s" % (vr(b + 8 + r), vr(b + 8 + r)))
+                        for r in range(4):
+                            e("v_mul_f32 %s, %s, %s" % (vr(b + r), vr(b + r), vr(b + 4 + r)))
+                        for r in range(4):
+                            e("v_mul_f32 %s, %s, %s" % (vr(b + r), vr(b + r), vr(b + 8 + r)))
+                        e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 8), vr(b), vr(b + 1)))
+                        e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 9), vr(b + 2), vr(b + 3)))
+                        e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 8, 2), (32 * il) * pitch + (32 * j + 8 * q) * 2))
+                continue
             for j in range(v.tn):
                 for q in range(4):
                     b = t + 6 * (k % 4)
@@ -582,16 +617,20 @@ def main():
     out.append("#define GMM_TILE_TR_STAGE %d" % TR_STAGE)
     out.append("#define GMM_TILE_STAGING_BYTES %d" % STAGE_BYTES)
     out.append("#define GMM_TILE_STAGES_SHORT %d" % STAGES_SHORT)
+    out.append("#define GMM_TILE_PITCH_ACT %d" % PITCH_ACT)
     for f16 in (0, 1):
-        for a_tr, b_tr, f32, tm, b_nt in [(a, b, f, t, n) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1) for n in (0, 1)]:
+        for a_tr, b_tr, f32, tm, b_nt, act in [(a, b, f, t, n, c) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1)
+                                               for n in (0, 1) for c in (0, 1)]:
             if tm != 4 and a_tr:
                 continue
             if b_nt and tm == 4:
                 continue      # only remainder tiles can be the sole reader of a B panel often enough to matter
-            v = Variant(a_tr, b_tr, f32, tm, f16, b_nt)
+            if act and (a_tr or f32):
+                continue      # the gated epilogue: K-contiguous first operand, 16-bit output
+            v = Variant(a_tr, b_tr, f32, tm, f16, b_nt, act)
             e = gen_variant(v)
             out.append("")
-            out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm, f16, b_nt))
+            out.append("template <> __device__ __forceinline__ void gmm_tile_asm<%d, %d, %d, %d, %d, %d, %d>(GmmTileRegs& r) {" % (a_tr, b_tr, f32, tm, f16, b_nt, act))
             out.append("  asm volatile(")
             out.append(e.text())
             out.append("      :")

@@ -104,6 +104,9 @@ int run(Problem& pr, hipStream_t stream) {
   const int forced = g_forced_path.load(std::memory_order_relaxed);
   const bool aligned = mfma_eligible(pr, lay, align);
   bool can_asm = aligned && asm_tile_eligible(pr, lay);
+  // the SwiGLU epilogue exists on the assembly tile only: K-contiguous first operand, 16-bit output, whole
+  // blocks of 64 gates + 64 partners
+  if (p.act && !(can_asm && lay.a_kc && pr.out_dtype == pr.in_dtype && (p.N & 127) == 0)) return GMM_ERR_UNSUPPORTED;
   if (p.gather) {
     // the assembly tile gathers rows of a K-contiguous first operand whose byte offsets fit 31 bits; the
     // register-staged MFMA kernel has no gather: everything else goes to the generic family
@@ -121,7 +124,7 @@ int run(Problem& pr, hipStream_t stream) {
     int cfg = g_forced_config.load(std::memory_order_relaxed);
     if (cfg == GMM_CFG_ASM_256x256 && !can_asm) return GMM_ERR_UNSUPPORTED;
     if (cfg < 0 || cfg >= GMM_CFG_COUNT) cfg = can_asm ? GMM_CFG_ASM_256x256 : GMM_CFG_REG_256x256;
-    if (p.gather && cfg != GMM_CFG_ASM_256x256) return GMM_ERR_UNSUPPORTED;
+    if ((p.gather || p.act) && cfg != GMM_CFG_ASM_256x256) return GMM_ERR_UNSUPPORTED;
     if (pr.in_dtype != GMM_DT_BF16 && cfg != GMM_CFG_ASM_256x256) return GMM_ERR_UNSUPPORTED;
     // the assembly tile stores 16-byte chunks: its tile columns start at multiples of 8 elements
     if (cfg == GMM_CFG_ASM_256x256 && p.jag == GMM_JAG_N) p.align = 8;
@@ -194,6 +197,22 @@ int gmm_2d3d_gather(const void* a, const int32_t* row_index, const void* b, void
   pr.p.a_rows = int32_t(a_rows);
   pr.in_dtype = in_dtype;
   pr.out_dtype = out_dtype;
+  return run(pr, static_cast<hipStream_t>(stream));
+}
+
+int gmm_2d3d_swiglu(const void* a, const int32_t* row_index, const void* b, void* out, const int32_t* offs, int32_t G,
+                    int64_t a_rows, int64_t M_total, int64_t N, int64_t K, int64_t a_sm, int64_t a_sk, int64_t b_sg,
+                    int64_t b_sk, int64_t b_sn, int64_t o_sm, int64_t o_sn, int32_t dtype, void* stream) {
+  if (!dims_ok(M_total, N, K) || !fits_i32(a_rows)) return GMM_ERR_BAD_ARGUMENT;
+  Problem pr{};
+  pr.p = GmmParams{a, b, out, offs, G, GMM_JAG_M, int32_t(M_total), int32_t(N), int32_t(K), 1,
+                   0, a_sm, a_sk, b_sg, b_sk, b_sn, 0, o_sm, o_sn, 0, 0};
+  pr.p.gather = row_index;
+  pr.p.a_rows = int32_t(row_index ? a_rows : M_total);
+  pr.p.act = 1;
+  pr.in_dtype = dtype;
+  pr.out_dtype = dtype;
+  if (g_forced_path.load(std::memory_order_relaxed) == GMM_PATH_GENERIC) return GMM_ERR_UNSUPPORTED;
   return run(pr, static_cast<hipStream_t>(stream));
 }
 

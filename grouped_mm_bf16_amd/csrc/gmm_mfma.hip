@@ -264,7 +264,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64, 1) gmm_mfma_kernel(cons
 // One wave per SIMD; tiles of 256, 128 and 64 rows share the launch when A is contiguous along K (a
 // column-major A has only the first): p.tall is the height of the tall tiles (256 or 128), p.shrt == 64
 // turns on the 64-row tiles for group remainders.
-template <int A_TR, int B_TR, int OUT_F32, int F16>
+template <int A_TR, int B_TR, int OUT_F32, int F16, int ACT = 0>
 __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
   constexpr int WAVES = 4;
   constexpr bool SHORT_TILES = !A_TR;
@@ -353,26 +353,28 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
         dsc.b.base = b + int64_t(k_begin) * ldb + n0;
         dsc.b.bytes = (int64_t(p.K - 1 - k_begin) * ldb + (p.N - n0)) * 2;
       }
-      dsc.c = C + (int64_t(g) * p.c_sg + int64_t(m0) * ldc + n0) * ESZ;
+      // SwiGLU epilogue: 256 columns of the product become 128 columns of the output
+      constexpr int CDIV = ACT ? 2 : 1;
+      dsc.c = C + (int64_t(g) * p.c_sg + int64_t(m0) * ldc + n0 / CDIV) * ESZ;
       dsc.ldc = ldc;
-      dsc.c_bytes = (int64_t(p.M - 1 - m0) * ldc + (p.N - n0)) * ESZ;
+      dsc.c_bytes = (int64_t(p.M - 1 - m0) * ldc + (p.N - n0) / CDIV) * ESZ;
       dsc.klen = k_hi > k_lo ? k_hi - k_begin : 0;
       dsc.khead = k_lo - k_begin;
       dsc.row_rel0 = m0 - m_lo;
       // rows past the tile's own height belong to the next tile of the group
       dsc.row_cnt = gmm_min(m_hi, m0 + rows) - m_lo;
-      dsc.col_lo = gmm_max(n_lo - n0, 0);
-      dsc.col_hi = gmm_min(n_hi - n0, GMM_TILE_N);
+      dsc.col_lo = gmm_max(n_lo - n0, 0) / CDIV;
+      dsc.col_hi = gmm_min(n_hi - n0, GMM_TILE_N) / CDIV;
       if constexpr (A_TR) {
         gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16>(dsc, lds_base, lane_j, wave);
       } else {
         // a short tile that holds all rows of its group is the only reader of its B panel
         const bool sole = m_hi - m_lo <= rows;
-        if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16>(dsc, lds_base, lane_j, wave);
-        else if (rows == 128 && !sole) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2, F16, 0>(dsc, lds_base, lane_j, wave);
-        else if (rows == 128) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2, F16, 1>(dsc, lds_base, lane_j, wave);
-        else if (!sole) gmm_tile_compute<A_TR, B_TR, OUT_F32, 1, F16, 0>(dsc, lds_base, lane_j, wave);
-        else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1, F16, 1>(dsc, lds_base, lane_j, wave);
+        if (rows == 256) gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16, 0, ACT>(dsc, lds_base, lane_j, wave);
+        else if (rows == 128 && !sole) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2, F16, 0, ACT>(dsc, lds_base, lane_j, wave);
+        else if (rows == 128) gmm_tile_compute<A_TR, B_TR, OUT_F32, 2, F16, 1, ACT>(dsc, lds_base, lane_j, wave);
+        else if (!sole) gmm_tile_compute<A_TR, B_TR, OUT_F32, 1, F16, 0, ACT>(dsc, lds_base, lane_j, wave);
+        else gmm_tile_compute<A_TR, B_TR, OUT_F32, 1, F16, 1, ACT>(dsc, lds_base, lane_j, wave);
       }
     }
     if (left <= BATCH) break;
@@ -383,6 +385,18 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
 template <int OUT_F32, int F16>
 int launch_asm(const GmmParams& p, GmmLayout lay, hipStream_t stream) {
   const dim3 grid(p.num_wg), block(256);
+  if (p.act) {
+    if constexpr (OUT_F32) {
+      return -1;
+    } else {
+      if (!lay.a_kc) return -1;
+      if (lay.b_kc)
+        hipLaunchKernelGGL((gmm_asm_kernel<0, 0, 0, F16, 1>), grid, block, 0, stream, p);
+      else
+        hipLaunchKernelGGL((gmm_asm_kernel<0, 1, 0, F16, 1>), grid, block, 0, stream, p);
+      return hipGetLastError() == hipSuccess ? 0 : 1;
+    }
+  }
   if (lay.a_kc && lay.b_kc)
     hipLaunchKernelGGL((gmm_asm_kernel<0, 0, OUT_F32, F16>), grid, block, 0, stream, p);
   else if (lay.a_kc && !lay.b_kc)

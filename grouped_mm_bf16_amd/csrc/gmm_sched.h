@@ -49,6 +49,8 @@ struct GmmParams {
   // (which then has `a_rows` rows); null: row r reads row r.
   const int32_t* gather;
   int32_t a_rows;
+  // 1: SwiGLU epilogue (assembly tile, jagged rows, 16-bit output): `c` has N / 2 columns, see gmm_tile.h
+  int32_t act;
 };
 
 GMM_HD int gmm_cdiv(int a, int b) { return (a + b - 1) / b; }

@@ -27,7 +27,9 @@ struct GmmTileRegs {
 // F16 = 1: A, B and a 16-bit output are fp16 instead of bf16 (same layouts, other MFMA and conversion).
 // B_NT = 1 (128- and 64-row tiles): B is copied with the non-temporal hint, for a tile that is the only
 // reader of its B panel (it then does not push panels that other tiles share out of the L2).
-template <int A_TR, int B_TR, int OUT_F32, int TM, int F16, int B_NT>
+// ACT = 1: SwiGLU epilogue.  Of every 128 columns of the product the first 64 are gates g and the last 64
+// their partners u; the tile stores silu(g) * u: 128 columns of a 16-bit output per 256-column tile.
+template <int A_TR, int B_TR, int OUT_F32, int TM, int F16, int B_NT, int ACT>
 __device__ __forceinline__ void gmm_tile_asm(GmmTileRegs& r);
 
 #include "gmm_tile_asm.inc"
@@ -94,7 +96,8 @@ struct GmmTileDesc {
   int khead;             // ... of which the first khead are before the group's range (0..7) and read as zero
   int row_rel0;          // m0 - m_lo   (may be negative: rows before m_lo are not stored)
   int row_cnt;           // m_hi - m_lo
-  int col_lo, col_hi;    // columns [col_lo, col_hi) of the tile are stored (relative to n0)
+  int col_lo, col_hi;    // columns [col_lo, col_hi) of the tile are stored (relative to n0; with the SwiGLU
+                         // epilogue: output columns relative to n0 / 2)
 };
 
 // NI = copy instructions per wave and K tile for this operand (8 for 256 rows, 2 per 64 rows).
@@ -143,9 +146,10 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, const GmmOp
   }
 }
 
-template <int A_TR, int B_TR, int OUT_F32, int TM = 4, int F16 = 0, int B_NT = 0>
+template <int A_TR, int B_TR, int OUT_F32, int TM = 4, int F16 = 0, int B_NT = 0, int ACT = 0>
 __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave) {
   static_assert(TM == 4 || !A_TR, "short tiles exist for a K-contiguous A only");
+  static_assert(!ACT || (!A_TR && !OUT_F32), "the SwiGLU epilogue: K-contiguous A, 16-bit output");
   constexpr int WROWS = 32 * TM;  // rows of the tile per wave row
   constexpr int B_BASE = GmmTileLayout<A_TR, TM>::b_base;
   const int wm = wave & 1, wn = wave >> 1;
@@ -173,12 +177,13 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   // Epilogue: the wave stages its block in LDS and reads it back row by row, 16 bytes per lane (see
   // gen_tile_asm.py).  ESZ bytes per element: a lane's chunk is NEL = 16 / ESZ columns, a row of the wave's
   // 128 columns takes LPR lanes, a read-back instruction covers 64 / LPR rows.
-  constexpr int ESZ = OUT_F32 ? 4 : 2, NEL = 16 / ESZ, LPR = 128 / NEL;
-  constexpr int EPITCH = OUT_F32 ? GMM_TILE_PITCH32 : GMM_TILE_PITCH;
+  constexpr int WCOLS = ACT ? 64 : 128;                   // output columns of a wave
+  constexpr int ESZ = OUT_F32 ? 4 : 2, NEL = 16 / ESZ, LPR = WCOLS / NEL;
+  constexpr int EPITCH = OUT_F32 ? GMM_TILE_PITCH32 : (ACT ? GMM_TILE_PITCH_ACT : GMM_TILE_PITCH);
   constexpr int STAGE_ROWS = OUT_F32 ? 32 : WROWS;        // rows a wave stages per pass
   int partial = 0;
   {
-    const int row_t = wm * WROWS + lane / LPR, col_t = wn * 128 + (lane % LPR) * NEL;
+    const int row_t = wm * WROWS + lane / LPR, col_t = wn * WCOLS + (lane % LPR) * NEL;
     const unsigned stage = lds_base + wave * (STAGE_ROWS * EPITCH);
     r.epi[0] = stage + (lane & 31) * EPITCH + 4 * ESZ * (lane >> 5);        // write: row lane % 32, columns 4 (lane / 32) ..
     r.epi[1] = stage + (lane / LPR) * EPITCH + (lane % LPR) * 16;           // read: row lane / LPR, chunk lane % LPR
@@ -227,5 +232,5 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   const int sc[8] = {nk, a_step, b_step, (int)lds_base, t.row_cnt, c_step, n_valid, wave | (flags << 8)};
 #pragma unroll
   for (int i = 0; i < 8; ++i) r.scal[i] = __builtin_amdgcn_readfirstlane(sc[i]);
-  gmm_tile_asm<A_TR, B_TR, OUT_F32, TM, F16, B_NT>(r);
+  gmm_tile_asm<A_TR, B_TR, OUT_F32, TM, F16, B_NT, ACT>(r);
 }

@@ -111,6 +111,45 @@ def grouped_mm_gathered(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tenso
     return out
 
 
+def interleave_gate_up(w_up: torch.Tensor) -> torch.Tensor:
+    """[E, H, 2I] with all gate columns first, then all partner ("up") columns  ->  the layout the fused SwiGLU
+    epilogue wants: in every block of 128 columns, 64 gate columns followed by their 64 partners.  I must be a
+    multiple of 64.  Done once, when the weights are loaded."""
+    E, H, N = w_up.shape
+    inner = N // 2
+    if N % 128:
+        raise RuntimeError("interleave_gate_up needs an inner size that is a multiple of 64")
+    g = w_up[..., :inner].reshape(E, H, inner // 64, 1, 64)
+    u = w_up[..., inner:].reshape(E, H, inner // 64, 1, 64)
+    return torch.cat([g, u], dim=3).reshape(E, H, N).contiguous()
+
+
+def grouped_mm_swiglu(a: torch.Tensor, row_index: torch.Tensor | None, b: torch.Tensor, offs: torch.Tensor,
+                      out: torch.Tensor | None = None) -> torch.Tensor:
+    """``swiglu(grouped_mm(a[row_index], b, offs))`` in one kernel, for ``b`` in the layout of
+    :func:`interleave_gate_up`; the [M_total, N] intermediate is never written.  Returns [M_total, N / 2].
+    Raises if the operands do not qualify for the fast path (see ``gmm_2d3d_swiglu`` in the C header)."""
+    _require_gpu(a, row_index, b, offs)
+    if a.dim() != 2 or b.dim() != 3 or a.dtype != b.dtype or a.size(1) != b.size(1):
+        raise RuntimeError("grouped_mm_swiglu takes a [R, K] and b [G, K, N] of one dtype")
+    if row_index is not None and (row_index.dtype != torch.int32 or row_index.dim() != 1 or not row_index.is_contiguous()):
+        raise RuntimeError("row_index has to be a contiguous 1D int32 tensor")
+    if offs.dtype != torch.int32 or offs.dim() != 1 or offs.numel() != b.size(0):
+        raise RuntimeError("offs has to be int32 [G]")
+    M = row_index.numel() if row_index is not None else a.size(0)
+    N = b.size(2)
+    if out is None:
+        out = torch.empty(M, N // 2, device=a.device, dtype=a.dtype)
+    lib = _lib.load()
+    with _guard(a):
+        rc = lib.gmm_2d3d_swiglu(a.data_ptr(), row_index.data_ptr() if row_index is not None else None, b.data_ptr(),
+                                 out.data_ptr(), offs.data_ptr(), offs.numel(), a.size(0), M, N, a.size(1),
+                                 a.stride(0), a.stride(1), b.stride(0), b.stride(1), b.stride(2), out.stride(0), out.stride(1),
+                                 _dtype_code(a.dtype), torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "grouped_mm_swiglu launch")
+    return out
+
+
 def moe_activation(h: torch.Tensor, kind: str = "swiglu", out: torch.Tensor | None = None) -> torch.Tensor:
     """``silu(h)`` or, for "swiglu", ``silu(h[:, :I]) * h[:, I:]`` with I = h.size(1) // 2 (fp32 arithmetic,
     one rounding).  h [R, I or 2I], bf16 or fp16, row-major."""
@@ -152,13 +191,16 @@ def moe_combine(y: torch.Tensor, routing: Routing, tokens: int, top_k: int, out:
 
 
 def moe_forward(x: torch.Tensor, router_logits: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, top_k: int,
-                activation: str = "swiglu", renormalize: bool = True) -> torch.Tensor:
+                activation: str = "swiglu", renormalize: bool = True, interleaved: bool = False) -> torch.Tensor:
     """One mixture-of-experts feed-forward layer.
 
     x [T, H]; router_logits [T, E]; w_up [E, H, I] ("silu") or [E, H, 2I] ("swiglu": gate columns first, then
     up columns); w_down [E, I, H].  Returns [T, H] in x's dtype:
     ``sum_j weight[t, j] * (act(x[t] @ w_up[e_tj]) @ w_down[e_tj])``.
     Intermediate results are rounded to x's dtype after each of the three stages, as separate layers would.
+
+    ``interleaved`` ("swiglu" only): ``w_up`` is in the layout of :func:`interleave_gate_up`; the activation then
+    runs inside the up projection's epilogue on the fp32 products (one rounding less, no [S, 2I] intermediate).
     """
     if x.dim() != 2 or router_logits.dim() != 2 or x.size(0) != router_logits.size(0):
         raise RuntimeError("x [T, H] and router_logits [T, E] must agree on T")
@@ -171,9 +213,14 @@ def moe_forward(x: torch.Tensor, router_logits: torch.Tensor, w_up: torch.Tensor
         raise RuntimeError("weight shapes do not chain: x [T, H], w_up [E, H, I or 2I], w_down [E, I, H]")
     T = x.size(0)
     routing = moe_route(router_logits, top_k, renormalize)
-    h = grouped_mm_gathered(x, routing.row_token, w_up, routing.offs)
-    act = moe_activation(h, activation)
-    del h
+    if interleaved:
+        if activation != "swiglu":
+            raise RuntimeError("interleaved weights go with the swiglu activation")
+        act = grouped_mm_swiglu(x, routing.row_token, w_up, routing.offs)
+    else:
+        h = grouped_mm_gathered(x, routing.row_token, w_up, routing.offs)
+        act = moe_activation(h, activation)
+        del h
     y = torch.empty(act.size(0), w_down.size(2), device=x.device, dtype=x.dtype)
     grouped_mm_2d3d(act, w_down, routing.offs, y)   # rows are already sorted by expert
     del act

@@ -72,6 +72,22 @@ int gmm_2d3d_gather(const void* a, const int32_t* row_index, const void* b, void
                     int64_t out_stride_m, int64_t out_stride_n,
                     int32_t in_dtype, int32_t out_dtype, void* stream);
 
+/* 2D x 3D with the SwiGLU activation applied to the product before it is stored (and, optionally, the row
+ * gather above: row_index may be NULL for rows already in place, a_rows is then ignored).
+ * b [G, K, N] holds, in every block of 128 columns, 64 gate columns followed by their 64 partner columns:
+ *   h = a[row_index] @ b[g]  (fp32),   out[r, 64 * blk + c] = silu(h[r, 128 * blk + c]) * h[r, 128 * blk + 64 + c],
+ * out [M_total, N / 2] in the input dtype (bf16 or fp16), rounded once: the intermediate h is never written.
+ * Assembly tile only: returns GMM_ERR_UNSUPPORTED unless a is contiguous along K, N % 128 == 0 and the
+ * operands meet the alignment rules of the fast path (16-byte aligned bases, leading dimensions multiples of
+ * 8 elements, out row-major).  No counterpart in the reference. */
+int gmm_2d3d_swiglu(const void* a, const int32_t* row_index, const void* b, void* out,
+                    const int32_t* offs, int32_t G, int64_t a_rows,
+                    int64_t M_total, int64_t N, int64_t K,
+                    int64_t a_stride_m, int64_t a_stride_k,
+                    int64_t b_stride_g, int64_t b_stride_k, int64_t b_stride_n,
+                    int64_t out_stride_m, int64_t out_stride_n,
+                    int32_t dtype, void* stream);
+
 /* 3D x 3D: out[g] = a[g] @ b[g]
  * a [G, M, K], b [G, K, N], out [G, M, N].
  * Replaces grouped_mm_3d3d(mat_a, mat_b, out), reference kernels.py:524-550. */

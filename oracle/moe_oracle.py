@@ -66,6 +66,18 @@ def activation(h: torch.Tensor, kind: str) -> torch.Tensor:
     raise ValueError(kind)
 
 
+def interleave_gate_up(w_up: torch.Tensor) -> torch.Tensor:
+    """Columns [gate_0..gate_{I-1} | up_0..up_{I-1}] -> per block of 128: 64 gates, then their 64 partners
+    (written with index arithmetic, not with the reshape the package uses)."""
+    n = w_up.shape[-1]
+    inner = n // 2
+    idx = torch.empty(n, dtype=torch.long)
+    for c in range(n):
+        blk, within = divmod(c, 128)
+        idx[c] = blk * 64 + within if within < 64 else inner + blk * 64 + (within - 64)
+    return w_up[..., idx]
+
+
 def combine(y: torch.Tensor, r: Routing, tokens: int, top_k: int) -> torch.Tensor:
     rows = r.token_rows.long().reshape(tokens, top_k)
     w = r.slot_weight.reshape(tokens, top_k)
@@ -76,11 +88,15 @@ def combine(y: torch.Tensor, r: Routing, tokens: int, top_k: int) -> torch.Tenso
 
 
 def moe_forward(x, logits, w_up, w_down, top_k: int, kind: str = "swiglu", renormalize: bool = True,
-                routing: Routing | None = None) -> torch.Tensor:
+                routing: Routing | None = None, fused: bool = False) -> torch.Tensor:
+    """w_up always in the plain [gate | up] layout.  fused: the activation sees the fp32 products (what the
+    fused epilogue does); else the products are rounded to the input dtype first (separate kernels)."""
     r = routing if routing is not None else route(logits, top_k, renormalize)
     xs = x[r.row_token.long()]
-    h = gmm.grouped_mm(xs, w_up, r.offs)
-    act = activation(h, kind)
+    if fused:
+        act = activation(gmm.grouped_mm(xs, w_up, r.offs, out_dtype=torch.float32), kind).to(x.dtype)
+    else:
+        act = activation(gmm.grouped_mm(xs, w_up, r.offs), kind)
     y = gmm.grouped_mm(act, w_down, r.offs)
     return combine(y, r, x.shape[0], top_k)
 

@@ -165,6 +165,58 @@ def test_gathered_product_on_views_and_large_sources():
     assert got.float().cpu().tolist() == [[16384.0] * 8, [0.0] * 8, [0.0] * 8]
 
 
+# ------------------------------------------------------------------ product with the SwiGLU epilogue
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("gather", [False, True])
+@pytest.mark.parametrize("dtype,K,N", [(torch.bfloat16, 136, 256), (torch.float16, 136, 384), (torch.bfloat16, 2048, 1536)])
+def test_fused_swiglu_product(dtype, K, N, gather, b_col):
+    """out = swiglu(a[idx] @ b[g]) from the fp32 accumulators, b in the interleaved layout; against the oracle
+    (activation of the fp32 product, one rounding) and against the two-kernel path on the same device."""
+    gen = torch.Generator().manual_seed(K + N)
+    G, M, S = len(SIZES), sum(SIZES), 401
+    a = rnd(gen, S if gather else M + 9, K, dtype=dtype)
+    w = rnd(gen, G, K, N, dtype=dtype, scale=K ** -0.5)                   # plain layout [gate | up]
+    idx = torch.randint(0, S, (M + 9,), generator=gen).to(torch.int32) if gather else None
+    offs = offs_of(SIZES)
+    wd = moe.interleave_gate_up(w.to(DEV))
+    if b_col:
+        wd = wd.transpose(1, 2).contiguous().transpose(1, 2)
+    out = torch.full((M + 9, N // 2), float("nan"), device=DEV, dtype=dtype)
+    moe.grouped_mm_swiglu(a.to(DEV), idx.to(DEV) if gather else None, wd, offs.to(DEV), out=out)
+    torch.cuda.synchronize()
+    assert K_.last_path() == "mfma"
+    got = out.cpu()
+    assert torch.isnan(got[M:].float()).all(), "rows past offs[-1] were written"
+    rows = a[idx.long()] if gather else a
+    h32 = oracle.grouped_mm(rows, w, offs, out_dtype=torch.float32)
+    want = moe_oracle.activation(h32[:M], "swiglu").to(dtype)
+    # |d swiglu| <= ~1.1 |dg| |u| + |du|: the product's bar carries over with the size of the partner
+    oracle.assert_close(got[:M], want, K)
+    ulp_like = (got[:M].float() - want.float()).abs() <= 2.0 ** -6 * want.float().abs() + 2e-3
+    assert ulp_like.float().mean() > 0.999
+    # two kernels: product rounded to 16 bits, then the activation kernel
+    h16 = torch.empty(M + 9, N, device=DEV, dtype=dtype)
+    if gather:
+        moe.grouped_mm_gathered(a.to(DEV), idx.to(DEV), w.to(DEV), offs.to(DEV), out=h16)
+    else:
+        K_.grouped_mm_2d3d(a.to(DEV), w.to(DEV), offs.to(DEV), h16)
+    two = moe.moe_activation(h16[:M], "swiglu").cpu()
+    oracle.assert_close(got[:M], two, K)
+
+
+def test_fused_swiglu_rejects_what_the_tile_cannot_do():
+    a = torch.zeros(64, 64, device=DEV, dtype=torch.bfloat16)
+    offs = torch.tensor([64], device=DEV, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        moe.grouped_mm_swiglu(a, None, torch.zeros(1, 64, 192, device=DEV, dtype=torch.bfloat16), offs)   # N % 128
+    with pytest.raises(RuntimeError, match="unsupported"):
+        moe.grouped_mm_swiglu(a.float(), None, torch.zeros(1, 64, 256, device=DEV), offs)                  # fp32
+    with pytest.raises(RuntimeError, match="unsupported"):
+        moe.grouped_mm_swiglu(a.t().contiguous().t(), None, torch.zeros(1, 64, 256, device=DEV, dtype=torch.bfloat16), offs)
+    with K_.forced_path("generic"), pytest.raises(RuntimeError, match="unsupported"):
+        moe.grouped_mm_swiglu(a, None, torch.zeros(1, 64, 256, device=DEV, dtype=torch.bfloat16), offs)
+
+
 # ------------------------------------------------------------------ activation, combine
 def ulp_close(got, want, dtype):
     """Equal up to one unit in the last place of the 16-bit type (fast exp and fused multiply-adds on the device)."""
@@ -231,10 +283,11 @@ def layer_case(seed, T, H, I, E, k, kind, dtype=torch.bfloat16, skew=0.0, wscale
             rnd(gen, E, I, H, dtype=dtype, scale=s_down))
 
 
-def run_layer(x, logits, w_up, w_down, k, kind, renorm=True):
-    got = moe.moe_forward(x.to(DEV), logits.to(DEV), w_up.to(DEV), w_down.to(DEV), k, kind, renorm)
+def run_layer(x, logits, w_up, w_down, k, kind, renorm=True, fused=False):
+    wu = moe.interleave_gate_up(w_up.to(DEV)) if fused else w_up.to(DEV)
+    got = moe.moe_forward(x.to(DEV), logits.to(DEV), wu, w_down.to(DEV), k, kind, renorm, interleaved=fused)
     torch.cuda.synchronize()
-    want = moe_oracle.moe_forward(x, logits, w_up, w_down, k, kind, renorm)
+    want = moe_oracle.moe_forward(x, logits, w_up, w_down, k, kind, renorm, fused=fused)
     # three stages, each within the grouped product's bar; the last contraction runs over I
     oracle.assert_close(got.cpu(), want, w_down.shape[1])
     # and as a whole far inside one rounding of the 16-bit type (differences come from rounding flips only)
@@ -249,6 +302,11 @@ def test_layer_small(T, H, I, E, k, kind):
     case = layer_case(T + E, T, H, I, E, k, kind)
     run_layer(*case, k, kind)
     run_layer(*case, k, kind, renorm=False)
+
+
+@pytest.mark.parametrize("T,H,I,E,k", [(130, 136, 256, 6, 2), (257, 256, 512, 16, 4), (64, 128, 64, 128, 8)])
+def test_layer_small_fused(T, H, I, E, k):
+    run_layer(*layer_case(T + E, T, H, I, E, k, "swiglu"), k, "swiglu", fused=True)
 
 
 def test_layer_fp16_and_dense_pin():
@@ -266,6 +324,7 @@ def test_layer_mixtral_size():
     logits[:, 0] += 1.0
     run_layer(x, logits, w_up, w_down, 2, "swiglu")
     assert K_.last_path() == "mfma"
+    run_layer(x, logits, w_up, w_down, 2, "swiglu", fused=True)
 
 
 def test_layer_fine_grained_size():
@@ -276,3 +335,4 @@ def test_layer_fine_grained_size():
     assert (sizes == 0).sum() > 10 and (sizes == 1).any() and (sizes < 16).sum() > 40
     run_layer(x, logits, w_up, w_down, 8, "swiglu")
     assert K_.last_path() == "mfma"
+    run_layer(x, logits, w_up, w_down, 8, "swiglu", fused=True)

@@ -125,3 +125,27 @@ def test_permuting_experts_permutes_nothing_a_caller_sees():
     a = moe.moe_forward(x, logits, w_up, w_down, k)
     b = moe.moe_forward(x, logits[:, p], w_up[p], w_down[p], k)
     assert torch.allclose(a, b, rtol=1e-5, atol=1e-5)
+
+
+def test_interleaved_layout_and_fused_rounding():
+    """The gate/partner interleave: block b of 128 columns = gate columns 64 b .. 64 b + 63, then their
+    partners; the package's reshape and the oracle's index arithmetic agree, and swiglu on the interleaved
+    product, taken block by block, equals swiglu on the plain one."""
+    from grouped_mm_bf16_amd.moe import interleave_gate_up
+    w = torch.arange(2 * 3 * 256, dtype=torch.float32).reshape(2, 3, 256)   # I = 128: columns 0..127 gates, 128..255 partners
+    il = moe.interleave_gate_up(w)
+    assert torch.equal(il, interleave_gate_up(w))
+    assert il[0, 0, :64].tolist() == list(range(0, 64)) and il[0, 0, 64:128].tolist() == list(range(128, 192))
+    assert il[0, 0, 128:192].tolist() == list(range(64, 128)) and il[0, 0, 192:].tolist() == list(range(192, 256))
+    gen = torch.Generator().manual_seed(3)
+    h = torch.randn(5, 256, generator=gen)
+    hi = moe.interleave_gate_up(h)
+    blocks = hi.reshape(5, 2, 2, 64)
+    fused = (torch.nn.functional.silu(blocks[:, :, 0]) * blocks[:, :, 1]).reshape(5, 128)
+    assert torch.equal(fused, moe.activation(h, "swiglu"))
+    # fused flag: same layer, one rounding less; with fp32 inputs the two coincide and match the dense formulation
+    x, logits = torch.randn(9, 16, generator=gen), torch.randn(9, 4, generator=gen)
+    w_up, w_down = torch.randn(4, 16, 128, generator=gen) * 0.2, torch.randn(4, 64, 16, generator=gen) * 0.2
+    a = moe.moe_forward(x, logits, w_up, w_down, 2, fused=True)
+    assert torch.allclose(a, moe.moe_forward(x, logits, w_up, w_down, 2), rtol=1e-6, atol=1e-6)
+    assert torch.allclose(a.double(), moe.moe_dense(x, logits, w_up, w_down, 2), rtol=1e-4, atol=1e-4)
