@@ -336,3 +336,59 @@ def test_layer_fine_grained_size():
     run_layer(x, logits, w_up, w_down, 8, "swiglu")
     assert K_.last_path() == "mfma"
     run_layer(x, logits, w_up, w_down, 8, "swiglu", fused=True)
+
+
+def test_layer_replays_from_a_captured_graph():
+    """The whole layer on static buffers -- routing through the entry point that allocates nothing, fused up
+    projection, down projection, combine -- captured once and replayed on new tokens and new router logits: the
+    routing, and with it `offs`, changes from replay to replay without the host ever seeing it.  Every replay
+    must equal the eager layer on the same inputs bit for bit, and the oracle within the bar."""
+    from grouped_mm_bf16_amd import _lib
+    lib = _lib.load()
+    T, H, I, E, k = 300, 256, 256, 16, 4
+    S = T * k
+    gen = torch.Generator().manual_seed(99)
+    w_up, w_down = rnd(gen, E, H, 2 * I, scale=H ** -0.5), rnd(gen, E, I, H, scale=2 * I ** -0.5)
+    w_il, w_dn = moe.interleave_gate_up(w_up.to(DEV)), w_down.to(DEV)
+    x_s = torch.zeros(T, H, device=DEV, dtype=torch.bfloat16)
+    lg_s = torch.zeros(T, E, device=DEV)
+    i32 = dict(device=DEV, dtype=torch.int32)
+    r = moe.Routing(torch.zeros(E, **i32), torch.zeros(S, **i32), torch.zeros(S, device=DEV), torch.zeros(S, **i32),
+                    torch.zeros(S, **i32))
+    act = torch.zeros(S, I, device=DEV, dtype=torch.bfloat16)
+    y = torch.zeros(S, H, device=DEV, dtype=torch.bfloat16)
+    out_s = torch.zeros(T, H, device=DEV, dtype=torch.bfloat16)
+
+    def layer():
+        rc = lib.gmm_moe_route_noalloc(lg_s.data_ptr(), E, _lib.DT_F32, T, E, k, 1, r.offs.data_ptr(), r.slot_expert.data_ptr(),
+                                       r.slot_weight.data_ptr(), r.row_token.data_ptr(), r.token_rows.data_ptr(),
+                                       torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        moe.grouped_mm_swiglu(x_s, r.row_token, w_il, r.offs, out=act)
+        K_.grouped_mm_2d3d(act, w_dn, r.offs, y)
+        moe.moe_combine(y, r, T, k, out=out_s)
+
+    layer()                                       # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            layer()
+    torch.cuda.current_stream().wait_stream(side)
+    seen = set()
+    for rep in range(3):
+        x, logits = rnd(gen, T, H), torch.randn(T, E, generator=gen) + rep * torch.randn(E, generator=gen)
+        x_s.copy_(x.to(DEV))
+        lg_s.copy_(logits.to(DEV))
+        out_s.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = out_s.clone()
+        seen.add(tuple(r.offs.tolist()))
+        eager = moe.moe_forward(x_s, lg_s, w_il, w_dn, k, interleaved=True)
+        torch.cuda.synchronize()
+        assert torch.equal(replayed.view(torch.int16), eager.view(torch.int16)), f"replay {rep} differs from eager"
+        oracle.assert_close(replayed.cpu(), moe_oracle.moe_forward(x, logits, w_up, w_down, k, fused=True), I)
+    assert len(seen) == 3, "the routing was meant to change between replays"
