@@ -459,7 +459,7 @@ def main():
     if args.workload in MOE_LAYERS:
         rec = run_moe(args.workload, args.steps, args.warmup, torch, dev)
         print(json.dumps({"metric": "MoE feed-forward layer, useful TFLOP/s of the two projections", "value": rec["tflops"],
-                          "unit": "TFLOP/s", "n_gpus": 1, "warmup": args.warmup, "ms_per_step": rec["ms"],
+                          "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": rec["ms"],
                           "higher_is_better": True, "dtype": "bf16", "data": "synthetic", "config": rec}))
         return
 

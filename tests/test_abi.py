@@ -64,3 +64,16 @@ def test_missing_library_is_a_loud_error(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.load()
+
+
+def test_route_workspace_size_is_host_arithmetic():
+    """gmm_moe_route_workspace_bytes needs no GPU: one int32 row of `experts` counters per sort workgroup of
+    at most 1024 slots, at most 256 workgroups; -1 for sizes the routing does not take."""
+    lib = _lib.load()
+    f = lib.gmm_moe_route_workspace_bytes
+    assert f(5000, 128, 8) == 40 * 128 * 4            # 40000 slots -> 40 workgroups
+    assert f(8192, 8, 2) == 16 * 8 * 4
+    assert f(1, 1, 1) == 4 and f(0, 8, 2) == 0
+    assert f(10 ** 7, 1023, 1) == 256 * 1023 * 4      # capped at 256 workgroups
+    assert f(-1, 8, 2) == -1 and f(8, 0, 1) == -1 and f(8, 1024, 1) == -1 and f(8, 8, 0) == -1
+    assert f(2 ** 30, 8, 2) == -1                     # tokens * top_k must stay below 2^31
