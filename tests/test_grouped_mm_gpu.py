@@ -171,6 +171,31 @@ def test_small_groups_on_every_tile_height(K, N, b_col, tall, shrt):
     check(out, a, b, offs_of(sizes), K, path="mfma")
 
 
+def test_output_larger_than_4_gib():
+    """70000 x 32768 bf16 output (4.6 GB): every tile's address arithmetic must be 64-bit up to the tile's
+    origin.  Rows on both sides of the 2 GiB and 4 GiB marks and of the group boundaries against the oracle."""
+    gen = torch.Generator().manual_seed(17)
+    sizes = [30000, 5, 39995]
+    m, K, N = sum(sizes), 64, 32768
+    a, b = rnd(gen, m, K), rnd(gen, len(sizes), K, N, scale=0.1)
+    offs = offs_of(sizes)
+    out = torch.empty(m, N, device=DEV, dtype=torch.bfloat16)
+    out[::997].fill_(float("nan"))
+    K_.grouped_mm_2d3d(a.to(DEV), b.to(DEV), offs.to(DEV), out)
+    torch.cuda.synchronize()
+    assert K_.last_path() == "mfma"
+    marks = [0, 255, 256, 29999, 30000, 30004, 30005, 32767, 32768, 32769, 65535, 65536, 65537, m - 257, m - 1]
+    rows = sorted(set(marks + list(range(0, m, 997))))
+    got = out[rows].cpu()
+    grp = torch.searchsorted(offs.long(), torch.tensor(rows), right=True)
+    for g in range(len(sizes)):
+        sel = (grp == g).nonzero().flatten()
+        if len(sel):
+            want = (a[[rows[i] for i in sel]].float() @ b[g].float()).to(torch.bfloat16)
+            oracle.assert_close(got[sel], want, K, what=f"group {g}")
+    del out
+
+
 def test_rows_past_the_last_offset_are_not_written():
     gen = torch.Generator().manual_seed(5)
     a, b = rnd(gen, 40, 64), rnd(gen, 2, 64, 48)
