@@ -305,10 +305,12 @@ def parity_check(w, out, offs, torch, oracle):
             oracle.assert_close(got[rows][:, s_:e_], want, w["k"], what=f"bench parity group {g}")
 
 
-def run_workload(name, steps, warmup, torch, dev, path="auto", wall=True):
+def run_workload(name, steps, warmup, torch, dev, path="auto", wall=True, settle_s=0.0):
     """Times one workload on tensors resident in HBM.  Returns (w, record): `record` has the wall-clock time
     over exactly `steps` steps (when `wall`), the per-launch kernel times from HIP events on the launch
-    stream, the roofline position and a parity flag."""
+    stream, the roofline position and a parity flag.  settle_s > 0 (the short runs of the `configs` object):
+    warm up for at least that long and time at least that long, whatever `steps` says -- a kernel of 0.15 ms
+    measured for a few milliseconds after the host-side set-up reads the clock ramp, not the kernel."""
     from grouped_mm_bf16_amd import kernels
     from oracle import grouped_mm_oracle as oracle
     w = make_workload(name, torch)
@@ -334,6 +336,15 @@ def run_workload(name, steps, warmup, torch, dev, path="auto", wall=True):
         for _ in range(warmup):
             step()
         torch.cuda.synchronize()
+        if settle_s > 0:
+            t0 = time.perf_counter()
+            n_done = 0
+            while time.perf_counter() - t0 < settle_s:
+                for _ in range(10):
+                    step()
+                torch.cuda.synchronize()
+                n_done += 10
+            steps = max(steps, n_done)      # as many timed steps as fitted into the warm-up interval
         ms_per_step = None
         if wall:
             # whole-job wall clock over exactly `steps` steps
@@ -342,7 +353,16 @@ def run_workload(name, steps, warmup, torch, dev, path="auto", wall=True):
                 step()
             torch.cuda.synchronize()
             ms_per_step = (time.perf_counter() - t0) / steps * 1e3
-        # per-launch kernel time: HIP events on the launch stream around each step
+        # kernel time per launch: one pair of HIP events on the launch stream around the timed region (back-to-back
+        # launches, as in the wall-clock loop); a second pass with a pair per step gives the spread (each of
+        # those readings also holds the gap that the event markers themselves put between two launches)
+        r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        r0.record()
+        for _ in range(steps):
+            step()
+        r1.record()
+        torch.cuda.synchronize()
+        k_avg = r0.elapsed_time(r1) / steps
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         for e0, e1 in evs:
             e0.record()
@@ -350,7 +370,6 @@ def run_workload(name, steps, warmup, torch, dev, path="auto", wall=True):
             e1.record()
         torch.cuda.synchronize()
         k_ms = [e0.elapsed_time(e1) for e0, e1 in evs]
-    k_avg = statistics.mean(k_ms)
     if w["bound"] == "hbm":
         achieved, peak, unit = w["bytes"] / (k_avg * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
     else:
@@ -358,11 +377,11 @@ def run_workload(name, steps, warmup, torch, dev, path="auto", wall=True):
     traffic, source = measured_traffic(name)
     roof = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
             "frac": round(achieved / peak, 4), "traffic": traffic, "traffic_source": source,
-            "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(k_ms), 4),
-            "kernel_ms_median": round(statistics.median(k_ms), 4),
+            "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min_single": round(min(k_ms), 4),
+            "kernel_ms_median_single": round(statistics.median(k_ms), 4),
             "algorithmic_flops": w["flops"], "algorithmic_bytes": w["bytes"]}
     del a, b, out
-    return w, {"ms_per_step": ms_per_step, "family": family, "roofline": roof, "parity": "ok"}
+    return w, {"ms_per_step": ms_per_step, "family": family, "roofline": roof, "parity": "ok", "steps": steps}
 
 
 MOE_LAYERS = {   # tokens, hidden, inner, experts, top_k
@@ -398,13 +417,18 @@ def run_moe(name, steps, warmup, torch, dev):
     oracle.assert_close(out[:n].cpu(), want, I, what=f"bench parity {name}")
     for _ in range(warmup):
         moe.moe_forward(x, logits, w_il, w_down, k, interleaved=True)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    for e0, e1 in evs:
-        e0.record()
-        moe.moe_forward(x, logits, w_il, w_down, k, interleaved=True)
-        e1.record()
     torch.cuda.synchronize()
-    ms = statistics.mean(e0.elapsed_time(e1) for e0, e1 in evs)
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.15:          # let the clocks settle after the host-side parity check
+        moe.moe_forward(x, logits, w_il, w_down, k, interleaved=True)
+        torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        moe.moe_forward(x, logits, w_il, w_down, k, interleaved=True)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
     flops = 2 * T * k * H * 2 * I + 2 * T * k * I * H
     return {"workload": f"MoE layer: {T} tokens, hidden {H}, inner {I} (SwiGLU in the up projection's epilogue), {E} experts, top {k}, bf16",
             "ms": round(ms, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 2), "bound": "mfma" if name == "moe_mixtral" else "hbm",
@@ -415,8 +439,8 @@ def run_moe(name, steps, warmup, torch, dev):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="mixtral",
                     choices=["mixtral", "readme", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "plain",
                              "copy", "mfma_only", "moe_mixtral", "moe_fine"])
@@ -489,14 +513,14 @@ def main():
         rec["configs"] = {}
         for name in ("readme", "batched", "batched_colmajor", "fine", "kgrouped"):
             try:
-                wi, ri = run_workload(name, 30, 10, torch, dev, args.path, wall=False)
+                wi, ri = run_workload(name, 30, 10, torch, dev, args.path, wall=False, settle_s=0.15)
                 k_avg = ri["roofline"]["kernel_ms_avg"]
                 rec["configs"][name] = {
                     "workload": wi["desc"], "kernel_family": ri["family"], "ms": k_avg,
                     "tflops": round(wi["flops"] / (k_avg * 1e-3) / 1e12, 2),
                     "gbs": round(wi["bytes"] / (k_avg * 1e-3) / 1e9, 1),
                     "bound": wi["bound"], "frac": ri["roofline"]["frac"] if wi["bound"] != "latency" else None,
-                    "traffic": ri["roofline"]["traffic"], "parity": ri["parity"], "steps": 30}
+                    "traffic": ri["roofline"]["traffic"], "parity": ri["parity"], "steps": ri["steps"]}
                 del wi
             except Exception as ex:   # a config that fails must not take the headline down with it
                 rec["configs"][name] = {"parity": "FAILED", "error": repr(ex)[:300]}
