@@ -28,6 +28,7 @@ if ROOT not in sys.path:
 METRIC = "TFLOP/s + % bf16 MFMA peak, 2D×3D MoE G=8 K=4096 N=14336, 1 GPU"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+SETTLE_S = 0.15            # seconds of untimed launches before warm-up, after the host-side parity check
 # workload -> tag in the name of its rocprofv3 summary under profiles/ (`..__<tag>.md`)
 PROFILE_TAG = {"readme": "readme_2d3d", "mixtral": "mixtral_2d3d", "fine": "fine_grained_2d3d", "batched": "batched_3d3d",
                "batched_colmajor": "batched_colmajor_3d3d", "kgrouped": "kgrouped_2d2d", "ngrouped": "ngrouped_3d2d"}
@@ -333,18 +334,21 @@ def run_workload(name, steps, warmup, torch, dev, path="auto", wall=True, settle
         torch.cuda.synchronize()
         parity_check(w, out, offs, torch, oracle)        # raises on a mismatch: nothing wrong gets timed
         family = kernels.last_path()
+        # The parity check above keeps the host busy for seconds while the GPU idles and its clocks fall; the
+        # first tens of milliseconds of work after that run 5-15 % slow.  Keep the GPU busy for SETTLE_S
+        # first (same launches, untimed), then do the `warmup` steps and time exactly `steps` steps.
+        t0 = time.perf_counter()
+        n_done = 0
+        while time.perf_counter() - t0 < max(settle_s, SETTLE_S):
+            for _ in range(10):
+                step()
+            torch.cuda.synchronize()
+            n_done += 10
+        if settle_s > 0:
+            steps = max(steps, n_done)      # short config runs: as many timed steps as fitted into that interval
         for _ in range(warmup):
             step()
         torch.cuda.synchronize()
-        if settle_s > 0:
-            t0 = time.perf_counter()
-            n_done = 0
-            while time.perf_counter() - t0 < settle_s:
-                for _ in range(10):
-                    step()
-                torch.cuda.synchronize()
-                n_done += 10
-            steps = max(steps, n_done)      # as many timed steps as fitted into the warm-up interval
         ms_per_step = None
         if wall:
             # whole-job wall clock over exactly `steps` steps
@@ -495,7 +499,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w["desc"], "kernel_family": r["family"],
-                   "pct_bf16_mfma_peak": round(tflops / PEAK_BF16_TFLOPS * 100, 2)},
+                   "pct_bf16_mfma_peak": round(tflops / PEAK_BF16_TFLOPS * 100, 2),
+                   "untimed_settle_s_before_warmup": SETTLE_S},
         "roofline": r["roofline"],
     }
     if args.library_comparator:
