@@ -108,6 +108,20 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, const GmmOp
                                                  gmm_v8i& head, gmm_v8i& full, gmm_v8i& tail) {
   const int ld = op.ld;
   int kk[8];
+  // gathered rows: all index loads first (one wait for the lot), then the range checks
+  int src[8];
+  if (!TR && op.gather) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int row = wave * (NI * 8) + i * 8 + (lane >> 3);
+      src[i] = op.gather[row < op.gather_n ? row : 0];
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int row = wave * (NI * 8) + i * 8 + (lane >> 3);
+      if (row >= op.gather_n || src[i] >= op.src_rows) src[i] = -1;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     if (i >= NI) { kk[i] = 0; full[i] = (int)GMM_OOB; continue; }
@@ -115,12 +129,8 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, const GmmOp
       const int row = wave * (NI * 8) + i * 8 + (lane >> 3);
       const int c = (lane & 7) ^ gmm_swz(row);
       kk[i] = c * 8;
-      int src = row;
-      if (op.gather) {
-        src = row < op.gather_n ? op.gather[row] : -1;
-        if (src >= op.src_rows) src = -1;
-      }
-      full[i] = src >= 0 ? src * ld * 2 + c * 16 : (int)GMM_OOB;
+      const int r = op.gather ? src[i] : row;
+      full[i] = r >= 0 ? r * ld * 2 + c * 16 : (int)GMM_OOB;
     } else {
       const int blk = wave * 8 + i;
       kk[i] = 8 * (blk >> 2) + (blk & 3) + 4 * (lane >> 5);
