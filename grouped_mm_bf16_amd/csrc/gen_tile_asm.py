@@ -51,6 +51,16 @@ import sys
 # copies (of the 16 per K tile and wave) issued in: step 3 right after the barrier, then steps 0, 1, 2
 # of the next K tile; the tile must have landed at that tile's barrier (end of its step 2).
 COPY_SCHEDULE = (8, 8, 0, 0)
+# Order of the copies of a K tile: B first.  B is the operand that streams from HBM (every group has its
+# own), A is re-read by every tile column and mostly comes out of the Infinity Cache: the copies issued
+# first have the most time to land.
+B_COPIES_FIRST = 1
+# L2 prefetch: in every K tile each wave issues one plain dword load per operand whose lanes touch the cache
+# lines of K tile kt + TOUCH_DIST (the result is discarded).  A direct-to-LDS copy can only be issued one K
+# tile ahead (two LDS buffers), which is less than the latency of HBM; the touches bring the lines into the
+# L2 ahead of time so that the copies hit.  0 = off.  TOUCH_OPS: which operands ("a", "b").
+TOUCH_DIST = 3
+TOUCH_OPS = "b"
 
 PITCH = 272           # bytes per staged row of 128 bf16 (256 + 16: shifts banks per row)
 PITCH32 = 528         # ... of 128 fp32 (512 + 16)
@@ -73,6 +83,8 @@ V_OOB = 188              # constant 0x80000000
 V_EPI2 = 190             # +0: store voffset whatever the chunk's validity, +1: mask of valid elements if partial
 V_BUFA, V_BUFB = 98, 110  # three-buffer variants: fragment addresses per (buffer, step), 12 + 12
 V_FIX = 196              # A first-chunk addr, A last-chunk addr, same for B (buffer 0)
+V_TOUCH = 192            # per-lane offsets of the L2 prefetch touches: +0 A, +1 B (K tile 0)
+V_TOUCH_DST = 96         # +0 / +1: where the touched dwords land (never read)
 V_CLOBBER = 122
 S_MASK = 28            # s[28:31] keep-mask of the first chunk of the k range, s[32:35] of the last chunk
 
@@ -120,11 +132,23 @@ class Variant:
         self.na = 2 * tm                 # copies of the A tile per wave and K tile
         self.nb = 8                      # ... of the B tile
         self.ncopy = self.na + self.nb
+        # issue index -> copy: A copies are 0 .. na - 1, B copies na .. ncopy - 1
+        self.order = list(range(self.ncopy))
+        if B_COPIES_FIRST:
+            self.order = list(range(self.na, self.ncopy)) + list(range(self.na))
+        # 256-row tiles only: the shorter ones have a third LDS buffer (copies two K tiles ahead) and are short of
+        # memory issue slots, not of prefetch distance (with touches the fine-grained workload lost 8 %)
+        self.touch = [op for op in "ab" if TOUCH_DIST and op in TOUCH_OPS and tm == 4]
+        self.nt = len(self.touch)
         c3 = (self.ncopy + 1) // 2
         self.sched = COPY_SCHEDULE if tm == 4 else (c3, self.ncopy - c3, 0, 0)
         # LDS buffers per operand: 2 for the 256-row tile (LDS is full), 3 for the shorter ones, whose K
         # tiles are short of MFMA work and would otherwise wait on memory latency every K tile
         self.stages = STAGES_SHORT if tm < 4 else 2
+        # The loop's wait leaves (stages - 1) sets of touches in flight; the prologue issues the sets for K
+        # tiles stages .. touch_dist - 1 after its copies, and the first wait of the loop must not count more
+        # sets than that: touch_dist - stages + 1 >= stages - 1.
+        self.touch_dist = max(TOUCH_DIST, 2 * self.stages - 2)
         self.a_stage = TR_STAGE if a_tr else (64 * tm * 128 if self.stages == 3 else KC_STAGE)
         self.b_stage = TR_STAGE if b_tr else KC_STAGE
         self.b_base = self.stages * self.a_stage   # LDS offset of B buffer 0
@@ -190,11 +214,12 @@ class Variant:
                 out.append("v_mfma_f32_32x32x16_%s %s, %s, %s, %s" % (self.dt, c, b, a, c))
         return out
 
-    # -- copy instruction n (0..15) of a K tile into buffer buf.
+    # -- copy instruction with issue index n (0..15) of a K tile into buffer buf.
     # s_tail / s_oob: SGPR pairs (lane masks all-ones / zero): use the tail offsets / kill the copy.
     # s_ka / s_kb: SGPRs with the tile's byte offsets along K for A and B.  which: "head" or "loop".
     def dma(self, n, buf, which, s_tail, s_oob, s_ka, s_kb, tmp):
         out = []
+        n = self.order[n]
         is_a = n < self.na
         i = n if is_a else n - self.na
         tr = self.a_tr if is_a else self.b_tr
@@ -223,6 +248,14 @@ class Variant:
         pol = " nt" if (self.b_nt and not is_a) else ""
         out.append("buffer_load_dwordx4 %s, %s, %s offen%s lds" % (src, sr(S_RA if is_a else S_RB, 4), sr(s_ka if is_a else s_kb), pol))
         return out
+
+
+def touch_group(v, op, s_mask, s_k, tmp):
+    """L2 prefetch of one operand's K tile: one dword per lane, each lane on another cache line (offsets from
+    the wrapper, v[V_TOUCH ..]); s_mask (SGPR pair): all-ones if that K tile exists, else nothing is fetched."""
+    i = 0 if op == "a" else 1
+    return ["v_cndmask_b32_e64 %s, %s, %s, %s" % (vr(tmp), vr(V_OOB), vr(V_TOUCH + i), sr(s_mask, 2)),
+            "buffer_load_dword %s, %s, %s, %s offen" % (vr(V_TOUCH_DST + i), vr(tmp), sr(S_RA if op == "a" else S_RB, 4), sr(s_k))]
 
 
 def m0_gaps(lines):
@@ -310,6 +343,7 @@ def gen_main(v, e, L):
     s_last = sT + 14                    # nk - 1
     s_zero = sT + 15
     s_waveA, s_waveB = sT + 20, sT + 21
+    s_tmask, s_kta, s_ktb = sT + 22, sT + 24, sT + 25   # L2 prefetch: "K tile exists" mask (pair), its K offsets
 
     def tile_masks(s_tile, s_tail, s_oob):
         # tail mask: tile == nk - 1 ; oob mask: tile >= nk
@@ -358,10 +392,22 @@ def gen_main(v, e, L):
         for n in range(v.ncopy if tix < S - 1 else c3):
             for ins in m0_gaps(v.dma(n, tix, "loop", s_tail, s_oob, s_ka, s_kb, V_TMP + (n % 8))):
                 e(ins)
+    # L2 prefetch of the K tiles that the loop's touches (tile kt + TOUCH_DIST) do not reach
+    n_pro_touch = 0
+    if v.nt:
+        for tix in range(S, v.touch_dist):
+            e("s_cmp_gt_u32 %s, %d" % (sr(S_NK), tix))
+            e("s_cselect_b64 %s, -1, 0" % sr(s_tmask, 2))
+            e("s_mul_i32 %s, %s, %d" % (sr(s_kta), sr(S_ASTEP), tix))
+            e("s_mul_i32 %s, %s, %d" % (sr(s_ktb), sr(S_BSTEP), tix))
+            for k, op in enumerate(v.touch):
+                for ins in touch_group(v, op, s_tmask, s_kta if op == "a" else s_ktb, V_TMP + 8 + k):
+                    e(ins)
+                n_pro_touch += 1
     # zero the accumulators while the copies fly
     for r in range(16 * v.tm * v.tn):
         e("v_accvgpr_write_b32 a%d, 0" % r)
-    e("s_waitcnt vmcnt(%d)" % ((S - 2) * v.ncopy + c3))
+    e("s_waitcnt vmcnt(%d)" % ((S - 2) * v.ncopy + c3 + n_pro_touch))
     e("s_barrier")
     has_kc = not (v.a_tr and v.b_tr)
     if has_kc:
@@ -409,6 +455,12 @@ def gen_main(v, e, L):
             tile_masks(s_t1, s_tail2, s_oob2)
         e("s_mul_i32 %s, %s, %s" % (sr(s_ka2), sr(s_t1), sr(S_ASTEP)))
         e("s_mul_i32 %s, %s, %s" % (sr(s_kb2), sr(s_t1), sr(S_BSTEP)))
+        if v.nt:
+            e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), v.touch_dist))
+            e("s_cmp_lt_u32 %s, %s" % (sr(s_t1), sr(S_NK)))
+            e("s_cselect_b64 %s, -1, 0" % sr(s_tmask, 2))
+            e("s_mul_i32 %s, %s, %s" % (sr(s_kta), sr(s_t1), sr(S_ASTEP)))
+            e("s_mul_i32 %s, %s, %s" % (sr(s_ktb), sr(s_t1), sr(S_BSTEP)))
         nb = (buf + 1) % S       # buffer of tile kt + 1
         cb = (buf + S - 1) % S   # buffer of tile kt + S - 1
         # step 0: MFMA set 0, read step 1 -> set 1, next copies of tile kt + S - 1
@@ -418,13 +470,17 @@ def gen_main(v, e, L):
         # step 1
         side = [[x] for x in v.frag_reads(buf, 2, 0)]
         side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)]
+        # the touches come after every copy of tile kt + S - 1 in issue order (c1 == c2 == 0), so the wait below
+        # can leave them in flight: they have until the next K tile's wait to land
+        assert c1 == 0 and c2 == 0
+        side += [touch_group(v, op, s_tmask, s_kta if op == "a" else s_ktb, V_TMP + 8 + k) for k, op in enumerate(v.touch)]
         interleave(e, v.mfmas(1), side, need, nreads)
         # step 2
         side = [[x] for x in v.frag_reads(buf, 3, 1)]
         side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)]
         interleave(e, v.mfmas(0), side, need, nreads)
         # tile kt+1 has landed for this wave; after the barrier for all, and `buf` is free
-        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % ((S - 2) * v.ncopy))
+        e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % ((S - 2) * (v.ncopy + v.nt) + v.nt))
         e("s_barrier")
         if not (v.a_tr and v.b_tr) and not fast:
             # the tile that has just landed is the last one and its last chunk is partial
@@ -636,7 +692,7 @@ def main():
             out.append("      :")
             out.append('      : "{v[128:135]}"(r.voa_head), "{v[136:143]}"(r.vob_head), "{v[144:151]}"(r.voa), "{v[152:159]}"(r.vob),')
             out.append('        "{v[160:167]}"(r.voa_tail), "{v[168:175]}"(r.vob_tail), "{v[176:179]}"(r.ra_addr), "{v[180:183]}"(r.rb_addr),')
-            out.append('        "{v[184:187]}"(r.epi), "{v[190:191]}"(r.epi2), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
+            out.append('        "{v[184:187]}"(r.epi), "{v[190:191]}"(r.epi2), "{v[192:193]}"(r.touch), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
             out.append("      : %s);" % clobbers(v))
             out.append("}")
     sys.stdout.write("\n".join(out) + "\n")

@@ -276,7 +276,7 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[LDS_MAX];
   __shared__ int32_t cum_tall[GMM_MAX_GROUPS + 1];
   __shared__ int32_t cum_short[GMM_MAX_GROUPS + 1];
-  __shared__ int32_t tiles[BATCH][10];
+  __shared__ int32_t tiles[BATCH][11];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
@@ -303,6 +303,7 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       int32_t* d = tiles[tid];
       d[0] = tile.g; d[1] = tile.m0; d[2] = tile.n0; d[3] = tile.m_lo; d[4] = tile.m_hi;
       d[5] = tile.n_lo; d[6] = tile.n_hi; d[7] = tile.k_lo; d[8] = tile.k_hi; d[9] = tile.rows;
+      d[10] = tile.share | (tile.sharers << 8);
     }
     __syncthreads();
     const int64_t left = (int64_t(total) - blockIdx.x + gridDim.x - 1) / gridDim.x - first;  // tiles of this workgroup from `first` on
@@ -320,6 +321,7 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       const int n_lo = __builtin_amdgcn_readfirstlane(d[5]), n_hi = __builtin_amdgcn_readfirstlane(d[6]);
       const int k_lo = __builtin_amdgcn_readfirstlane(d[7]), k_hi = __builtin_amdgcn_readfirstlane(d[8]);
       const int rows = __builtin_amdgcn_readfirstlane(d[9]);
+      const int shr = __builtin_amdgcn_readfirstlane(d[10]);
       // the copies move 16-byte chunks along K for an operand that is contiguous along K
       const int k_begin = (A_TR && B_TR) ? k_lo : (k_lo & ~7);
       const uint16_t* a = A + int64_t(g) * p.a_sg;
@@ -365,6 +367,8 @@ __global__ void __launch_bounds__(256, 1) gmm_asm_kernel(const GmmParams p) {
       dsc.row_cnt = gmm_min(m_hi, m0 + rows) - m_lo;
       dsc.col_lo = gmm_max(n_lo - n0, 0) / CDIV;
       dsc.col_hi = gmm_min(n_hi - n0, GMM_TILE_N) / CDIV;
+      dsc.share = shr & 0xff;
+      dsc.sharers = shr >> 8;
       if constexpr (A_TR) {
         gmm_tile_compute<A_TR, B_TR, OUT_F32, 4, F16>(dsc, lds_base, lane_j, wave);
       } else {

@@ -172,12 +172,15 @@ struct GmmTile {
   int32_t n_lo, n_hi;    // columns that may be stored
   int32_t k_lo, k_hi;    // contraction range that contributes
   int32_t rows;          // height of the tile (0: the kernel's only height)
+  int32_t share, sharers;  // the tile is number `share` of the `sharers` tiles of its band that read the same
+                           // panel of the second operand at the same time (L2 prefetch shares); 0 sharers: none
 };
 
 GMM_HD GmmTile gmm_make_tile(const GmmParams& p, int g, int lo, int hi, int mt, int nt, int bm, int bn) {
   GmmTile t;
   t.g = g;
   t.rows = 0;
+  t.share = 0; t.sharers = 0;
   t.m0 = mt * bm; t.m_lo = 0; t.m_hi = p.M;
   t.n0 = nt * bn; t.n_lo = 0; t.n_hi = p.N;
   t.k_lo = 0; t.k_hi = p.K;
@@ -202,5 +205,10 @@ GMM_HD GmmTile gmm_make_tile2(const GmmParams& p, int g, int lo, int hi, int cls
   GmmTile t = gmm_make_tile(p, g, lo, hi, 0, nt, p.tall, bn);
   t.m0 += m_off;
   t.rows = cls == 0 ? p.tall : rem_rows;
+  if (cls == 0) {
+    const int first = (mt / GMM_BAND) * GMM_BAND;
+    t.share = mt - first;
+    t.sharers = gmm_min(n_tall - first, GMM_BAND);
+  }
   return t;
 }

@@ -17,6 +17,7 @@ struct GmmTileRegs {
   gmm_v4i epi;                 // epilogue: per-lane addresses (see gen_tile_asm.py)
   gmm_v2i epi2;                // bf16 epilogue: store offset of the lane's chunk whatever its validity; mask of
                                // its valid elements when only some of them are (a group boundary inside it)
+  gmm_v2i touch;               // L2 prefetch: byte offset of the cache line this lane touches in K tile 0 of A, of B (or out of range)
   gmm_v4i fix;                 // LDS addresses of this thread's row in the first / last k chunk (A, A, B, B)
   gmm_v8i masks;               // keep-masks of the first and of the last 16-byte k chunk
   gmm_v4i rsrc_a, rsrc_b, rsrc_c;
@@ -98,6 +99,7 @@ struct GmmTileDesc {
   int row_cnt;           // m_hi - m_lo
   int col_lo, col_hi;    // columns [col_lo, col_hi) of the tile are stored (relative to n0; with the SwiGLU
                          // epilogue: output columns relative to n0 / 2)
+  int share, sharers;    // L2 prefetch of B: this tile touches share number `share` of `sharers` (0: none)
 };
 
 // NI = copy instructions per wave and K tile for this operand (8 for 256 rows, 2 per 64 rows).
@@ -209,6 +211,21 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
     r.epi2[0] = off;
     r.epi2[1] = mask == FULL ? 0 : mask;
     partial = ((t.col_lo | t.col_hi) & (NEL - 1)) ? 1 : 0;
+  }
+  // L2 prefetch touches of B.  A K tile of B is 256 cache lines of 128 bytes: one per row when B is
+  // contiguous along K, else four per k row (64 k rows of 512 bytes).  The tile rows of a band run at the
+  // same time on one XCD and read the same B panel: each of the `sharers` tiles touches its own share of the
+  // lines, a quarter of it per wave, so every line is requested once, early, and the copies of all sharers hit.
+  {
+    int off_b = (int)GMM_OOB;
+    if (t.sharers > 0) {
+      const int per_tile = (256 + t.sharers - 1) / t.sharers, per_wave = (per_tile + 3) >> 2;
+      const int idx = wave * per_wave + lane, line = t.share * per_tile + idx;
+      if (lane < per_wave && idx < per_tile && line < 256)
+        off_b = B_TR ? (line >> 2) * t.b.ld * 2 + (line & 3) * 128 : line * t.b.ld * 2;
+    }
+    r.touch[0] = (int)GMM_OOB;
+    r.touch[1] = off_b;
   }
   const int c_step = (64 / LPR) * t.ldc * ESZ;
   const int n_valid = 0;
