@@ -12,7 +12,7 @@ import threading
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libgrouped_mm_hip.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # enum gmm_path / gmm_dtype / gmm_status of the header
 PATH_AUTO, PATH_GENERIC, PATH_MFMA = 0, 1, 2
@@ -25,12 +25,13 @@ _i32, _i64, _vp = ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p
 SIGNATURES = {
     "gmm_abi_version": (ctypes.c_int, []),
     "gmm_status_string": (ctypes.c_char_p, [ctypes.c_int]),
-    "gmm_2d3d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),
-    "gmm_2d3d_gather": (ctypes.c_int, [_vp] * 5 + [_i32] + [_i64] * 4 + [_i64] * 7 + [_i32, _i32, _vp]),
+    "gmm_workspace_bytes": (_i64, []),
+    "gmm_2d3d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp, _i64, _vp]),
+    "gmm_2d3d_gather": (ctypes.c_int, [_vp] * 5 + [_i32] + [_i64] * 4 + [_i64] * 7 + [_i32, _i32, _vp, _i64, _vp]),
     "gmm_2d3d_swiglu": (ctypes.c_int, [_vp] * 5 + [_i32] + [_i64] * 4 + [_i64] * 7 + [_i32, _vp]),
-    "gmm_3d3d": (ctypes.c_int, [_vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 9 + [_i32, _i32, _vp]),
-    "gmm_2d2d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),
-    "gmm_3d2d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp]),
+    "gmm_3d3d": (ctypes.c_int, [_vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 9 + [_i32, _i32, _vp, _i64, _vp]),
+    "gmm_2d2d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp, _i64, _vp]),
+    "gmm_3d2d": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32] + [_i64] * 3 + [_i64] * 7 + [_i32, _i32, _vp, _i64, _vp]),
     "gmm_moe_route_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "gmm_moe_route": (ctypes.c_int, [_vp, _i64, _i32, _i64, _i64, _i64, _i32] + [_vp] * 5 + [_vp, _i64, _vp]),
     "gmm_moe_route_noalloc": (ctypes.c_int, [_vp, _i64, _i32, _i64, _i64, _i64, _i32] + [_vp] * 5 + [_vp]),
@@ -43,7 +44,10 @@ SIGNATURES = {
     "gmm_set_xcd_remap": (ctypes.c_int, [ctypes.c_int]),
     "gmm_host_tile_list": (_i64, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _i64]),
     "gmm_host_tile_list2": (_i64, [_vp] + [_i32] * 11 + [_vp, _i64]),
+    "gmm_host_tile_list3": (_i64, [_vp] + [_i32] * 13 + [_vp, _i64]),
     "gmm_set_tile_heights": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
+    "gmm_set_tail_split": (ctypes.c_int, [ctypes.c_int]),
+    "gmm_set_group_major": (ctypes.c_int, [ctypes.c_int]),
     "gmm_diag_mfma_rate": (ctypes.c_int, [_vp, _i64, _vp, _i64, _i32, _i32, _vp, _vp]),
 }
 

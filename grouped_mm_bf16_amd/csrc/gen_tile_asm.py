@@ -124,8 +124,9 @@ class Variant:
         act: SwiGLU epilogue -- of each 128 columns the first 64 are gates and the last 64 their partners;
         the tile stores silu(gate) * partner, 128 columns of a 16-bit output per 256 columns of the product."""
         self.a_tr, self.b_tr, self.out_f32, self.tm, self.f16, self.b_nt = a_tr, b_tr, out_f32, tm, f16, b_nt
-        self.act = act
-        assert not (act and (out_f32 or a_tr))
+        self.act = act == 1
+        self.partial = act == 2      # fp32 partial tile of a tile cut along K: stored through to memory (sc1)
+        assert not (self.act and (out_f32 or a_tr)) and not (self.partial and (not out_f32 or b_nt))
         self.dt = "f16" if f16 else "bf16"   # element type of A, B and of a 16-bit output
         assert tm in (1, 2, 4) and (tm == 4 or not a_tr)
         self.tn = 4                      # 32-column MFMA blocks per wave (the wave grid is 2 x 2)
@@ -153,7 +154,7 @@ class Variant:
         self.b_stage = TR_STAGE if b_tr else KC_STAGE
         self.b_base = self.stages * self.a_stage   # LDS offset of B buffer 0
         self.name = "%s%s_%s_%s_m%d%s%s" % ("t" if a_tr else "k", "t" if b_tr else "k", self.dt, "f32" if out_f32 else self.dt, 64 * tm,
-                                            "_bnt" if b_nt else "", "_swiglu" if act else "")
+                                            "_bnt" if b_nt else "", "_swiglu" if act == 1 else ("_partial" if act == 2 else ""))
 
     def acc(self, i, j):
         return (self.tn * i + j) * 16
@@ -626,7 +627,9 @@ def gen_epilogue(v, e, L):
             e("v_cndmask_b32 %s, %s, %s, vcc" % (vr(vsel), vr(V_OOB), vr(voff)))
             # non-temporal: the output is written once and not read by this kernel; kept out of the way, it does
             # not push operand panels that other workgroups are about to share out of the L2
-            e("buffer_store_dwordx4 %s, %s, %s, 0 offen nt" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4)))
+            # a partial tile is read by the workgroup that adds the parts up, maybe on another XCD: written through
+            # at device scope
+            e("buffer_store_dwordx4 %s, %s, %s, 0 offen %s" % (vr(regs[r % depth], 4), vr(vsel), sr(S_RC, 4), "sc1" if v.partial else "nt"))
             e("s_bitcmp1_b32 %s, 2" % sr(S_T + 18))
             e("s_cbranch_scc0 L_nopart%d_%s" % (nstore, L))
             for el in range(nel):
@@ -676,13 +679,15 @@ def main():
     out.append("#define GMM_TILE_PITCH_ACT %d" % PITCH_ACT)
     for f16 in (0, 1):
         for a_tr, b_tr, f32, tm, b_nt, act in [(a, b, f, t, n, c) for a in (0, 1) for b in (0, 1) for f in (0, 1) for t in (4, 2, 1)
-                                               for n in (0, 1) for c in (0, 1)]:
+                                               for n in (0, 1) for c in (0, 1, 2)]:
             if tm != 4 and a_tr:
                 continue
             if b_nt and tm == 4:
                 continue      # only remainder tiles can be the sole reader of a B panel often enough to matter
-            if act and (a_tr or f32):
+            if act == 1 and (a_tr or f32):
                 continue      # the gated epilogue: K-contiguous first operand, 16-bit output
+            if act == 2 and (not f32 or b_nt):
+                continue      # partial tiles: fp32, ordinary B copies
             v = Variant(a_tr, b_tr, f32, tm, f16, b_nt, act)
             e = gen_variant(v)
             out.append("")

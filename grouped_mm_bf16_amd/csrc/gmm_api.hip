@@ -15,6 +15,8 @@ std::atomic<int> g_forced_config{-1};
 std::atomic<int> g_xcd_remap{1};
 std::atomic<int> g_forced_tall{-1};   // -1 auto, else 256 / 128
 std::atomic<int> g_forced_short{-1};  // -1 auto, 0 off, 64 on
+std::atomic<int> g_group_major{-1};   // -1 auto, 0 tall tiles of all groups first, 1 group by group
+std::atomic<int> g_tail_split{1};     // 0: ignore the workspace (no tile is cut along K)
 thread_local int t_last_path = 0;
 thread_local int t_last_config = -1;
 
@@ -42,6 +44,17 @@ struct Problem {
   GmmParams p;
   int in_dtype, out_dtype;
 };
+
+// Caller's workspace -> split parameters: the header must fit, the slots must be 16-byte aligned.
+void set_workspace(GmmParams& p, void* ws, int64_t bytes) {
+  p.ws = nullptr;
+  p.ws_parts = 0;
+  if (!g_tail_split.load(std::memory_order_relaxed)) return;
+  if (!ws || !aligned16(ws) || bytes < GMM_WS_HEADER + 2 * int64_t(GMM_WS_SLOT)) return;
+  const int64_t parts = (bytes - GMM_WS_HEADER) / GMM_WS_SLOT;
+  p.ws = ws;
+  p.ws_parts = int32_t(parts > 4096 ? 4096 : parts);   // 32-bit byte offsets from a tile's first slot
+}
 
 // Decide whether the MFMA family can take the call, and with which operand layouts.
 bool mfma_eligible(const Problem& pr, GmmLayout& lay, int& align) {
@@ -141,6 +154,13 @@ int run(Problem& pr, hipStream_t stream) {
       if (lay.a_kc && (ft == 256 || ft == 128)) p.tall = ft;
       if (lay.a_kc && (fs == 0 || fs == 64)) p.shrt = fs;
     }
+    // Launch order: group by group in the fine-grained regime (many small groups: a group's remainder tile
+    // then reads the second operand while its tall tiles have it in the caches; +4 % there), otherwise all
+    // tall tiles first (longest first balances the rounds; the down projection loses 1 % group by group).
+    {
+      const int fo = g_group_major.load(std::memory_order_relaxed);
+      p.group_major = fo >= 0 ? fo : (p.tall == 128 ? 1 : 0);
+    }
     rc = gmm_launch_mfma(p, lay, pr.in_dtype, pr.out_dtype, cfg, cus, stream);
     t_last_path = GMM_PATH_MFMA;
     t_last_config = cfg;
@@ -161,6 +181,11 @@ extern "C" {
 
 int gmm_abi_version(void) { return GMM_ABI_VERSION; }
 
+int64_t gmm_workspace_bytes(void) {
+  const int cus = device_cus();
+  return cus > 0 ? GMM_WS_HEADER + 2 * int64_t(cus) * GMM_WS_SLOT : 0;
+}
+
 const char* gmm_status_string(int status) {
   switch (status) {
     case GMM_OK: return "ok";
@@ -174,20 +199,22 @@ const char* gmm_status_string(int status) {
 
 int gmm_2d3d(const void* a, const void* b, void* out, const int32_t* offs, int32_t G, int64_t M_total,
              int64_t N, int64_t K, int64_t a_sm, int64_t a_sk, int64_t b_sg, int64_t b_sk, int64_t b_sn,
-             int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* stream) {
+             int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* workspace,
+             int64_t workspace_bytes, void* stream) {
   if (!dims_ok(M_total, N, K)) return GMM_ERR_BAD_ARGUMENT;
   Problem pr{};
   pr.p = GmmParams{a, b, out, offs, G, GMM_JAG_M, int32_t(M_total), int32_t(N), int32_t(K), 1,
                    0, a_sm, a_sk, b_sg, b_sk, b_sn, 0, o_sm, o_sn, 0, 0};
   pr.in_dtype = in_dtype;
   pr.out_dtype = out_dtype;
+  set_workspace(pr.p, workspace, workspace_bytes);
   return run(pr, static_cast<hipStream_t>(stream));
 }
 
 int gmm_2d3d_gather(const void* a, const int32_t* row_index, const void* b, void* out, const int32_t* offs, int32_t G,
                     int64_t a_rows, int64_t M_total, int64_t N, int64_t K, int64_t a_sm, int64_t a_sk, int64_t b_sg,
-                    int64_t b_sk, int64_t b_sn, int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype,
-                    void* stream) {
+                    int64_t b_sk, int64_t b_sn, int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* workspace,
+                    int64_t workspace_bytes, void* stream) {
   if (!dims_ok(M_total, N, K) || !fits_i32(a_rows)) return GMM_ERR_BAD_ARGUMENT;
   if (!row_index && M_total > 0 && G > 0 && N > 0) return GMM_ERR_BAD_ARGUMENT;
   Problem pr{};
@@ -197,6 +224,7 @@ int gmm_2d3d_gather(const void* a, const int32_t* row_index, const void* b, void
   pr.p.a_rows = int32_t(a_rows);
   pr.in_dtype = in_dtype;
   pr.out_dtype = out_dtype;
+  set_workspace(pr.p, workspace, workspace_bytes);
   return run(pr, static_cast<hipStream_t>(stream));
 }
 
@@ -218,13 +246,15 @@ int gmm_2d3d_swiglu(const void* a, const int32_t* row_index, const void* b, void
 
 int gmm_3d3d(const void* a, const void* b, void* out, int32_t G, int64_t M, int64_t N, int64_t K,
              int64_t a_sg, int64_t a_sm, int64_t a_sk, int64_t b_sg, int64_t b_sk, int64_t b_sn,
-             int64_t o_sg, int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* stream) {
+             int64_t o_sg, int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* workspace,
+             int64_t workspace_bytes, void* stream) {
   if (!dims_ok(M, N, K)) return GMM_ERR_BAD_ARGUMENT;
   Problem pr{};
   pr.p = GmmParams{a, b, out, nullptr, G, GMM_JAG_NONE, int32_t(M), int32_t(N), int32_t(K), 1,
                    a_sg, a_sm, a_sk, b_sg, b_sk, b_sn, o_sg, o_sm, o_sn, 0, 0};
   pr.in_dtype = in_dtype;
   pr.out_dtype = out_dtype;
+  set_workspace(pr.p, workspace, workspace_bytes);
   // the tile count G * tiles must fit an int32
   if (G > 0 && M > 0 && N > 0) {
     const int64_t tiles = int64_t(G) * ((M + 63) / 64) * ((N + 63) / 64);
@@ -235,25 +265,29 @@ int gmm_3d3d(const void* a, const void* b, void* out, int32_t G, int64_t M, int6
 
 int gmm_2d2d(const void* a, const void* b, void* out, const int32_t* offs, int32_t G, int64_t M, int64_t N,
              int64_t K_total, int64_t a_sm, int64_t a_sk, int64_t b_sk, int64_t b_sn, int64_t o_sg,
-             int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* stream) {
+             int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* workspace,
+             int64_t workspace_bytes, void* stream) {
   if (!dims_ok(M, N, K_total)) return GMM_ERR_BAD_ARGUMENT;
   Problem pr{};
   pr.p = GmmParams{a, b, out, offs, G, GMM_JAG_K, int32_t(M), int32_t(N), int32_t(K_total), 1,
                    0, a_sm, a_sk, 0, b_sk, b_sn, o_sg, o_sm, o_sn, 0, 0};
   pr.in_dtype = in_dtype;
   pr.out_dtype = out_dtype;
+  set_workspace(pr.p, workspace, workspace_bytes);
   return run(pr, static_cast<hipStream_t>(stream));
 }
 
 int gmm_3d2d(const void* a, const void* b, void* out, const int32_t* offs, int32_t G, int64_t M,
              int64_t N_total, int64_t K, int64_t a_sg, int64_t a_sm, int64_t a_sk, int64_t b_sk, int64_t b_sn,
-             int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* stream) {
+             int64_t o_sm, int64_t o_sn, int32_t in_dtype, int32_t out_dtype, void* workspace,
+             int64_t workspace_bytes, void* stream) {
   if (!dims_ok(M, N_total, K)) return GMM_ERR_BAD_ARGUMENT;
   Problem pr{};
   pr.p = GmmParams{a, b, out, offs, G, GMM_JAG_N, int32_t(M), int32_t(N_total), int32_t(K), 1,
                    a_sg, a_sm, a_sk, 0, b_sk, b_sn, 0, o_sm, o_sn, 0, 0};
   pr.in_dtype = in_dtype;
   pr.out_dtype = out_dtype;
+  set_workspace(pr.p, workspace, workspace_bytes);
   return run(pr, static_cast<hipStream_t>(stream));
 }
 
@@ -265,6 +299,8 @@ int gmm_last_path(void) { return t_last_path; }
 int gmm_set_mfma_config(int config) { return g_forced_config.exchange(config); }
 int gmm_last_mfma_config(void) { return t_last_config; }
 int gmm_set_xcd_remap(int on) { return g_xcd_remap.exchange(on ? 1 : 0); }
+int gmm_set_group_major(int mode) { return g_group_major.exchange(mode < 0 ? -1 : (mode ? 1 : 0)); }
+int gmm_set_tail_split(int on) { return g_tail_split.exchange(on ? 1 : 0); }
 int gmm_set_tile_heights(int tall, int shrt) {
   const int prev_tall = g_forced_tall.exchange(tall), prev_short = g_forced_short.exchange(shrt);
   return ((prev_tall + 1) << 16) | ((prev_short + 1) & 0xffff);
@@ -305,13 +341,15 @@ int64_t gmm_host_tile_list(const int32_t* offs_host, int32_t G, int32_t jagged, 
   return total;
 }
 
-int64_t gmm_host_tile_list2(const int32_t* offs_host, int32_t G, int32_t jagged, int32_t M, int32_t N, int32_t K,
-                            int32_t tall, int32_t shrt, int32_t tile_n, int32_t align, int32_t xcd_remap,
-                            int32_t num_workgroups, int32_t* records, int64_t capacity) {
-  if (G < 0 || jagged < 0 || jagged > 3 || tall <= 0 || shrt < 0 || tile_n <= 0 || align <= 0)
+// Shared by gmm_host_tile_list2 / 3: the launch order of the assembly tile's kernel, run on the host.
+static int64_t host_tile_list23(const int32_t* offs_host, int32_t G, int32_t jagged, int32_t M, int32_t N, int32_t K,
+                                int32_t tall, int32_t shrt, int32_t tile_n, int32_t align, int32_t xcd_remap,
+                                int32_t num_workgroups, int32_t max_parts, int32_t group_major, int32_t width,
+                                int32_t* records, int64_t capacity) {
+  if (G < 0 || jagged < 0 || jagged > 3 || tall <= 0 || shrt < 0 || tile_n <= 0 || align <= 0 || max_parts < 0)
     return -GMM_ERR_BAD_ARGUMENT;
   if (jagged != GMM_JAG_NONE && (!offs_host || G < 1 || G >= GMM_MAX_GROUPS)) return -GMM_ERR_BAD_ARGUMENT;
-  if (xcd_remap && (num_workgroups <= 0 || num_workgroups % 8)) return -GMM_ERR_BAD_ARGUMENT;
+  if ((xcd_remap || max_parts) && (num_workgroups <= 0 || num_workgroups % 8)) return -GMM_ERR_BAD_ARGUMENT;
   GmmParams p{};
   p.offs = offs_host;
   p.G = G; p.jag = jagged; p.M = M; p.N = N; p.K = K; p.align = align; p.tall = tall; p.shrt = shrt;
@@ -322,26 +360,73 @@ int64_t gmm_host_tile_list2(const int32_t* offs_host, int32_t G, int32_t jagged,
     if (jagged != GMM_JAG_NONE) gmm_group_range(offs_host, g, extent, lo, hi);
     gmm_split_rows(gmm_group_rows(jagged, lo, hi, M, align), tall, shrt, n_tall, n_short, rem_rows);
     const int tn = gmm_group_tile_cols(jagged, lo, hi, N, align, tile_n);
-    ct[g + 1] = ct[g] + n_tall * tn;
-    cs[g + 1] = cs[g] + n_short * tn;
+    ct[g + 1] = ct[g] + n_tall * tn + (group_major ? n_short * tn : 0);
+    cs[g + 1] = cs[g] + (group_major ? 0 : n_short * tn);
   }
-  const int total_tall = ct[G], total = ct[G] + cs[G];
+  const int total_tall = ct[G], total_tiles = ct[G] + cs[G];
+  // the split of the last round, as gmm_asm_kernel decides it
+  const int nk = gmm_cdiv(K, 64);
+  int nparts = 1, tail = 0;
+  if (max_parts > 0 && jagged != GMM_JAG_K) {
+    nparts = gmm_tail_split(total_tiles, num_workgroups, nk, max_parts);
+    if (nparts > 1) tail = total_tiles % num_workgroups;
+  }
+  // round-robin tiles in launch order, then the parts in ticket order (which workgroup runs a part is
+  // decided at run time)
+  const int split_base = total_tiles - tail, total = split_base + tail * nparts;
   for (int t = 0; t < total; ++t) {
-    const int tt = xcd_remap ? gmm_xcd_remap(t, total, num_workgroups) : t;
-    const int cls = tt < total_tall ? 0 : 1;
+    int tt, part = 0;
+    const bool is_part = t >= split_base;
+    if (!is_part) {
+      tt = xcd_remap ? gmm_xcd_remap(t, split_base, num_workgroups) : t;
+    } else {
+      part = (t - split_base) / tail;
+      tt = split_base + (t - split_base) % tail;
+    }
+    int cls = tt < total_tall ? 0 : 1;
     const int tc = cls ? tt - total_tall : tt;
     const std::vector<int32_t>& cum = cls ? cs : ct;
     const int g = gmm_find_group(cum.data(), G, tc);
-    int lo = 0, hi = 0;
+    int lo = 0, hi = 0, local = tc - cum[g];
     if (jagged != GMM_JAG_NONE) gmm_group_range(offs_host, g, extent, lo, hi);
-    const GmmTile tile = gmm_make_tile2(p, g, lo, hi, cls, tc - cum[g], tile_n);
+    if (group_major) {
+      // one table: a group's tall tiles, then its remainder tiles
+      int n_tall, n_short, rem_rows;
+      gmm_split_rows(gmm_group_rows(jagged, lo, hi, M, align), tall, shrt, n_tall, n_short, rem_rows);
+      const int tall_tiles = n_tall * gmm_group_tile_cols(jagged, lo, hi, N, align, tile_n);
+      if (local >= tall_tiles) { cls = 1; local -= tall_tiles; }
+    }
+    GmmTile tile = gmm_make_tile2(p, g, lo, hi, cls, local, tile_n);
+    if (is_part) {
+      int kt0, kt1;
+      gmm_part_ktiles(nk, nparts, part, kt0, kt1);
+      tile.k_lo = kt0 * 64;
+      tile.k_hi = gmm_min(kt1 * 64, K);
+    }
     if (t < capacity && records) {
-      int32_t* r = records + int64_t(t) * 10;
+      int32_t* r = records + int64_t(t) * width;
       r[0] = tile.g; r[1] = tile.m0; r[2] = tile.n0; r[3] = tile.m_lo; r[4] = tile.m_hi;
       r[5] = tile.n_lo; r[6] = tile.n_hi; r[7] = tile.k_lo; r[8] = tile.k_hi; r[9] = tile.rows;
+      if (width >= 12) { r[10] = part; r[11] = is_part ? nparts : 1; }
     }
   }
   return total;
+}
+
+int64_t gmm_host_tile_list2(const int32_t* offs_host, int32_t G, int32_t jagged, int32_t M, int32_t N, int32_t K,
+                            int32_t tall, int32_t shrt, int32_t tile_n, int32_t align, int32_t xcd_remap,
+                            int32_t num_workgroups, int32_t* records, int64_t capacity) {
+  return host_tile_list23(offs_host, G, jagged, M, N, K, tall, shrt, tile_n, align, xcd_remap, num_workgroups, 0, 0, 10,
+                          records, capacity);
+}
+
+int64_t gmm_host_tile_list3(const int32_t* offs_host, int32_t G, int32_t jagged, int32_t M, int32_t N, int32_t K,
+                            int32_t tall, int32_t shrt, int32_t tile_n, int32_t align, int32_t xcd_remap,
+                            int32_t num_workgroups, int32_t max_parts, int32_t group_major, int32_t* records,
+                            int64_t capacity) {
+  if (group_major && jagged == GMM_JAG_NONE) group_major = 0;   // batches are all alike: one order
+  return host_tile_list23(offs_host, G, jagged, M, N, K, tall, shrt, tile_n, align, xcd_remap, num_workgroups,
+                          max_parts, group_major ? 1 : 0, 12, records, capacity);
 }
 
 }  // extern "C"

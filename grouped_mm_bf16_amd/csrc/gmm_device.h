@@ -117,8 +117,8 @@ __device__ __forceinline__ int gmm_build_tile_table2(const GmmParams& p, int bn,
       ct = n_tall * tn;
       cs = n_short * tn;
     }
-    cum_tall[g + 1] = ct;
-    cum_short[g + 1] = cs;
+    cum_tall[g + 1] = p.group_major ? ct + cs : ct;
+    cum_short[g + 1] = p.group_major ? 0 : cs;
   }
   if (tid == 0) { cum_tall[0] = 0; cum_short[0] = 0; }
   __syncthreads();
@@ -126,16 +126,26 @@ __device__ __forceinline__ int gmm_build_tile_table2(const GmmParams& p, int bn,
   gmm_scan_table<NT>(cum_short);
   __syncthreads();
   total_tall = cum_tall[p.G];
-  return total_tall + cum_short[p.G];
+  return total_tall + cum_short[p.G];   // group-major order: everything is in the first table
 }
 
 // Tile id -> tile, per lane (ids differ between lanes).
 __device__ __forceinline__ GmmTile gmm_locate_tile2(const GmmParams& p, const int32_t* cum_tall, const int32_t* cum_short,
                                                     int total_tall, int t, int bn) {
-  const int cls = t < total_tall ? 0 : 1;
+  int cls = t < total_tall ? 0 : 1;
   const int tc = cls ? t - total_tall : t;
   int g, local, lo = 0, hi = 0;
-  if (p.jag == GMM_JAG_NONE) {
+  if (p.group_major && p.jag != GMM_JAG_NONE) {
+    // one table: a group's tall tiles, then its remainder tiles
+    g = gmm_find_group(cum_tall, p.G, t);
+    local = t - cum_tall[g];
+    gmm_group_range(p.offs, g, p.jag == GMM_JAG_M ? p.M : (p.jag == GMM_JAG_N ? p.N : p.K), lo, hi);
+    int n_tall, n_short, rem_rows;
+    gmm_split_rows(gmm_group_rows(p.jag, lo, hi, p.M, p.align), p.tall, p.shrt, n_tall, n_short, rem_rows);
+    const int tall_tiles = n_tall * gmm_group_tile_cols(p.jag, lo, hi, p.N, p.align, bn);
+    cls = local < tall_tiles ? 0 : 1;
+    if (cls) local -= tall_tiles;
+  } else if (p.jag == GMM_JAG_NONE) {
     int n_tall, n_short, rem_rows;
     gmm_split_rows(p.M, p.tall, p.shrt, n_tall, n_short, rem_rows);
     const int per = (cls ? n_short : n_tall) * gmm_cdiv(p.N, bn);

@@ -51,11 +51,52 @@ struct GmmParams {
   int32_t a_rows;
   // 1: SwiGLU epilogue (assembly tile, jagged rows, 16-bit output): `c` has N / 2 columns, see gmm_tile.h
   int32_t act;
+  // Split of the last, partly filled round of the launch along K (assembly tile; see gmm_tail_split): fp32
+  // partial tiles go to `ws` (GMM_WS_HEADER bytes of arrival counters that are zero between launches, then
+  // `ws_parts` slots of GMM_WS_SLOT bytes); null / 0: no split.
+  void* ws;
+  int32_t ws_parts;
+  // Launch order of tiles of different heights.  0: all tall tiles of all groups, then all remainder tiles.
+  // 1: group by group, a group's remainder tiles right after its tall tiles, while the group's second
+  // operand is still in the Infinity Cache.
+  int32_t group_major;
 };
+
+constexpr int GMM_WS_HEADER = 4096;          // 1024 int32: arrival counters, one per tile of the split round, ...
+constexpr int GMM_WS_SLOT = 256 * 256 * 4;   // one fp32 partial tile
+constexpr int GMM_SPLIT_MAX = 8;             // most parts a tile is cut into
+constexpr int GMM_SPLIT_PART_NK = 48;        // K tiles (of 64) a part aims at: long enough to carry its extra fp32
+                                             // store and the reduction, short enough to even out the tail
+constexpr int GMM_WS_TICKET = 1020;          // header words beyond the arrival counters: next part to hand out,
+constexpr int GMM_WS_EXITED = 1021;          // workgroups that have left the ticket loop
 
 GMM_HD int gmm_cdiv(int a, int b) { return (a + b - 1) / b; }
 GMM_HD int gmm_min(int a, int b) { return a < b ? a : b; }
 GMM_HD int gmm_max(int a, int b) { return a > b ? a : b; }
+
+// A persistent launch deals `total` tiles to W workgroups round by round; the last round holds
+// tail = total % W tiles and leaves W - tail workgroups idle for a whole tile.  When the workspace allows,
+// every tile of that round is cut along K into S parts (its K tiles split evenly) that any free workgroup
+// takes from a ticket counter; each part stores an fp32 partial tile, and the part that arrives last adds the
+// partials in part order (the sum does not depend on timing) and stores the output.  Returns S (1: no
+// split): parts of about GMM_SPLIT_PART_NK K tiles, at most GMM_SPLIT_MAX per tile, as the workspace allows;
+// no split when the contraction is short or the round is more than three quarters full (the parts' extra
+// stores and the reduction then cost what the idle workgroups would).  nk = K tiles per tile (the same for
+// every tile: not for a jagged contraction).
+GMM_HD int gmm_tail_split(int total, int W, int nk, int max_parts) {
+  const int tail = total % W;
+  if (tail == 0 || tail > GMM_WS_TICKET || 4 * tail > 3 * W || nk < 2 * GMM_SPLIT_PART_NK) return 1;
+  int S = (nk + GMM_SPLIT_PART_NK / 2) / GMM_SPLIT_PART_NK;
+  S = gmm_min(S, GMM_SPLIT_MAX);
+  S = gmm_min(S, max_parts / tail);
+  return S < 2 ? 1 : S;
+}
+
+// K tiles [first, last) of part `part` of S of a tile with nk K tiles.
+GMM_HD void gmm_part_ktiles(int nk, int S, int part, int& first, int& last) {
+  first = int(int64_t(part) * nk / S);
+  last = int(int64_t(part + 1) * nk / S);
+}
 
 // [lo, hi) of group g along the jagged dimension, clamped into [0, extent] and
 // made non-decreasing so that malformed offsets can never index out of bounds.
@@ -172,6 +213,8 @@ struct GmmTile {
   int32_t n_lo, n_hi;    // columns that may be stored
   int32_t k_lo, k_hi;    // contraction range that contributes
   int32_t rows;          // height of the tile (0: the kernel's only height)
+  int32_t part, nparts;    // part `part` of `nparts` along K (nparts 1: the whole tile); tail_idx: index of the tile
+  int32_t tail_idx;        // in the split round (its arrival counter)
   int32_t share, sharers;  // the tile is number `share` of the `sharers` tiles of its band that read the same
                            // panel of the second operand at the same time (L2 prefetch shares); 0 sharers: none
 };
@@ -181,6 +224,7 @@ GMM_HD GmmTile gmm_make_tile(const GmmParams& p, int g, int lo, int hi, int mt, 
   t.g = g;
   t.rows = 0;
   t.share = 0; t.sharers = 0;
+  t.part = 0; t.nparts = 1; t.tail_idx = 0;
   t.m0 = mt * bm; t.m_lo = 0; t.m_hi = p.M;
   t.n0 = nt * bn; t.n_lo = 0; t.n_hi = p.N;
   t.k_lo = 0; t.k_hi = p.K;

@@ -28,6 +28,8 @@ struct GmmTileRegs {
 // F16 = 1: A, B and a 16-bit output are fp16 instead of bf16 (same layouts, other MFMA and conversion).
 // B_NT = 1 (128- and 64-row tiles): B is copied with the non-temporal hint, for a tile that is the only
 // reader of its B panel (it then does not push panels that other tiles share out of the L2).
+// ACT = 2: the tile is a partial sum (a part of a tile cut along K): fp32, stored through to memory at
+// device scope (sc1), so that a workgroup on another XCD can read it without anybody flushing an L2.
 // ACT = 1: SwiGLU epilogue.  Of every 128 columns of the product the first 64 are gates g and the last 64
 // their partners u; the tile stores silu(g) * u: 128 columns of a 16-bit output per 256-column tile.
 template <int A_TR, int B_TR, int OUT_F32, int TM, int F16, int B_NT, int ACT>
@@ -161,7 +163,8 @@ __device__ __forceinline__ void gmm_copy_offsets(int lane, int wave, const GmmOp
 template <int A_TR, int B_TR, int OUT_F32, int TM = 4, int F16 = 0, int B_NT = 0, int ACT = 0>
 __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned lds_base, int lane, int wave) {
   static_assert(TM == 4 || !A_TR, "short tiles exist for a K-contiguous A only");
-  static_assert(!ACT || (!A_TR && !OUT_F32), "the SwiGLU epilogue: K-contiguous A, 16-bit output");
+  static_assert(ACT != 1 || (!A_TR && !OUT_F32), "the SwiGLU epilogue: K-contiguous A, 16-bit output");
+  static_assert(ACT != 2 || (OUT_F32 && !B_NT), "partial tiles are fp32");
   constexpr int WROWS = 32 * TM;  // rows of the tile per wave row
   constexpr int B_BASE = GmmTileLayout<A_TR, TM>::b_base;
   const int wm = wave & 1, wn = wave >> 1;
@@ -189,9 +192,9 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   // Epilogue: the wave stages its block in LDS and reads it back row by row, 16 bytes per lane (see
   // gen_tile_asm.py).  ESZ bytes per element: a lane's chunk is NEL = 16 / ESZ columns, a row of the wave's
   // 128 columns takes LPR lanes, a read-back instruction covers 64 / LPR rows.
-  constexpr int WCOLS = ACT ? 64 : 128;                   // output columns of a wave
+  constexpr int WCOLS = ACT == 1 ? 64 : 128;                   // output columns of a wave
   constexpr int ESZ = OUT_F32 ? 4 : 2, NEL = 16 / ESZ, LPR = WCOLS / NEL;
-  constexpr int EPITCH = OUT_F32 ? GMM_TILE_PITCH32 : (ACT ? GMM_TILE_PITCH_ACT : GMM_TILE_PITCH);
+  constexpr int EPITCH = OUT_F32 ? GMM_TILE_PITCH32 : (ACT == 1 ? GMM_TILE_PITCH_ACT : GMM_TILE_PITCH);
   constexpr int STAGE_ROWS = OUT_F32 ? 32 : WROWS;        // rows a wave stages per pass
   int partial = 0;
   {

@@ -37,6 +37,29 @@ def _require_gpu(*tensors) -> None:
             raise RuntimeError("grouped_mm_bf16 is GPU-only (CUDA/HIP); CPU tensors are not supported")
 
 
+# One workspace per (device, stream): launches on one stream run one after the other, so they can share it;
+# launches on different streams may overlap and must not.  Allocated on first use and kept (the library leaves
+# the arrival counters at its head zero after every launch).
+_workspaces: dict = {}
+
+
+def workspace(device: torch.device, stream: int):
+    """(pointer, bytes) of the split workspace for launches on `stream` of `device`, or (None, 0) when none
+    can be had: inside a stream capture no new workspace is allocated (a captured allocation would belong to
+    the graph's memory pool), so a stream first used under capture launches without one."""
+    key = (device.index, stream)
+    ws = _workspaces.get(key)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None, 0
+        nbytes = _lib.load().gmm_workspace_bytes()
+        if nbytes <= 0:
+            return None, 0
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws.data_ptr(), ws.numel()
+
+
 def _launch_now(variant: int, a: torch.Tensor, b: torch.Tensor, offs: Optional[torch.Tensor],
                 out: torch.Tensor) -> None:
     lib = _lib.load()
@@ -48,22 +71,23 @@ def _launch_now(variant: int, a: torch.Tensor, b: torch.Tensor, offs: Optional[t
         stream = torch.cuda.current_stream().cuda_stream
         pa, pb, po = a.data_ptr(), b.data_ptr(), out.data_ptr()
         poffs = offs.data_ptr() if offs is not None else None
+        ws, ws_bytes = workspace(a.device, stream)
         if variant == V_2D3D:
             rc = lib.gmm_2d3d(pa, pb, po, poffs, offs.numel(), a.size(0), b.size(2), a.size(1),
                               a.stride(0), a.stride(1), b.stride(0), b.stride(1), b.stride(2),
-                              out.stride(0), out.stride(1), in_dt, out_dt, stream)
+                              out.stride(0), out.stride(1), in_dt, out_dt, ws, ws_bytes, stream)
         elif variant == V_3D3D:
             rc = lib.gmm_3d3d(pa, pb, po, a.size(0), a.size(1), b.size(2), a.size(2),
                               a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1), b.stride(2),
-                              out.stride(0), out.stride(1), out.stride(2), in_dt, out_dt, stream)
+                              out.stride(0), out.stride(1), out.stride(2), in_dt, out_dt, ws, ws_bytes, stream)
         elif variant == V_2D2D:
             rc = lib.gmm_2d2d(pa, pb, po, poffs, offs.numel(), a.size(0), b.size(1), a.size(1),
                               a.stride(0), a.stride(1), b.stride(0), b.stride(1),
-                              out.stride(0), out.stride(1), out.stride(2), in_dt, out_dt, stream)
+                              out.stride(0), out.stride(1), out.stride(2), in_dt, out_dt, ws, ws_bytes, stream)
         elif variant == V_3D2D:
             rc = lib.gmm_3d2d(pa, pb, po, poffs, offs.numel(), a.size(1), b.size(1), a.size(2),
                               a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1),
-                              out.stride(0), out.stride(1), in_dt, out_dt, stream)
+                              out.stride(0), out.stride(1), in_dt, out_dt, ws, ws_bytes, stream)
         else:
             raise RuntimeError(f"unknown variant {variant}")
     _lib.check(rc, "grouped_mm launch")
@@ -152,6 +176,20 @@ def forced_tile_heights(tall: int, shrt: int):
         yield
     finally:
         lib.gmm_set_tile_heights((prev >> 16) - 1, (prev & 0xffff) - 1)
+
+
+@contextlib.contextmanager
+def tail_split(on: bool):
+    """Inside the block launches do (True) or do not (False) cut the tiles of a sparse last round along the
+    contraction.  A cut tile adds its fp32 partial sums in a fixed order, so results are reproducible either
+    way, but they differ in the last bit from the uncut tile's: tests that compare two launches bit for bit
+    across different tile lists switch the split off."""
+    lib = _lib.load()
+    prev = lib.gmm_set_tail_split(1 if on else 0)
+    try:
+        yield
+    finally:
+        lib.gmm_set_tail_split(prev)
 
 
 def last_path() -> str:

@@ -17,7 +17,7 @@ from typing import NamedTuple
 
 import torch
 
-from . import _lib
+from . import _lib, kernels
 from .kernels import _dtype_code, _require_gpu, grouped_mm_2d3d
 
 ACTIVATIONS = {"silu": 0, "swiglu": 1}
@@ -103,10 +103,12 @@ def grouped_mm_gathered(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tenso
         return out.zero_()
     lib = _lib.load()
     with _guard(a):
+        stream = torch.cuda.current_stream().cuda_stream
+        ws, ws_bytes = kernels.workspace(a.device, stream)
         rc = lib.gmm_2d3d_gather(a.data_ptr(), row_index.data_ptr(), b.data_ptr(), out.data_ptr(), offs.data_ptr(),
                                  offs.numel(), a.size(0), M, N, a.size(1), a.stride(0), a.stride(1),
                                  b.stride(0), b.stride(1), b.stride(2), out.stride(0), out.stride(1),
-                                 _dtype_code(a.dtype), _dtype_code(out.dtype), torch.cuda.current_stream().cuda_stream)
+                                 _dtype_code(a.dtype), _dtype_code(out.dtype), ws, ws_bytes, stream)
     _lib.check(rc, "grouped_mm_gathered launch")
     return out
 

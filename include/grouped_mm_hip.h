@@ -14,6 +14,9 @@
  *     dimension (the first group starts at 0); it is read on the device only;
  *   - in_dtype / out_dtype are gmm_dtype values; out_dtype is in_dtype or
  *     GMM_DT_F32;
+ *   - `workspace` / `workspace_bytes`: optional device memory (NULL / 0: none) that lets a launch whose
+ *     last round of tiles would leave most of the chip idle cut those tiles along the contraction (see
+ *     gmm_workspace_bytes below); the library itself never allocates;
  *   - `stream` is a hipStream_t (NULL = the default stream);
  *   - the return value is a gmm_status; nothing is thrown across the boundary.
  *   - elements that no group owns (rows / columns at or beyond offs[G-1]) are
@@ -28,7 +31,7 @@
 extern "C" {
 #endif
 
-#define GMM_ABI_VERSION 2
+#define GMM_ABI_VERSION 3
 
 enum gmm_status {
   GMM_OK = 0,
@@ -47,6 +50,22 @@ enum gmm_path { GMM_PATH_AUTO = 0, GMM_PATH_GENERIC = 1, GMM_PATH_MFMA = 2 };
 int gmm_abi_version(void);
 const char* gmm_status_string(int status);
 
+/* Workspace of the launchers below.  The kernels deal output tiles to one workgroup per compute unit, round
+ * by round; when the last round holds far fewer tiles than there are compute units (a down projection
+ * 16384 x 14336 -> 4096 has 4.25 rounds of tiles on 256 units) its tiles are cut along the contraction into
+ * up to 8 parts, every part stores an fp32 partial tile in the workspace, and the part that arrives last adds
+ * the partials in part order and stores the output: the result does not depend on timing and is rounded
+ * once.  Layout: 4096 bytes of arrival counters, then slots of 262144 bytes (one fp32 tile each); the more
+ * slots, the more freedom to split.  gmm_workspace_bytes() returns the size the library can make full use
+ * of on the current device (4096 + 2 * compute units * 262144; 128 MiB on MI355X); a smaller workspace
+ * limits the split, less than 4096 + 2 * 262144 bytes (or NULL) turns it off.  Rules for the caller:
+ *   - 16-byte aligned; the first 4096 bytes zero before the first launch that uses it (the kernels leave
+ *     them zero, so one hipMemset after allocation is enough); the rest need not be initialised;
+ *   - launches that may run at the same time (different streams) need different workspaces.
+ * The reference has no counterpart (its launches create one program per tile, reference
+ * kernels.py:636-659, and leave the balancing to the hardware dispatcher). */
+int64_t gmm_workspace_bytes(void);
+
 /* 2D x 3D: out[s_g:e_g, :] = a[s_g:e_g, :] @ b[g]   (rows jagged)
  * a [M_total, K], b [G, K, N], out [M_total, N].
  * Replaces grouped_mm_2d3d(mat_a, mat_b, offs, out), reference kernels.py:583-686. */
@@ -55,7 +74,8 @@ int gmm_2d3d(const void* a, const void* b, void* out, const int32_t* offs, int32
              int64_t a_stride_m, int64_t a_stride_k,
              int64_t b_stride_g, int64_t b_stride_k, int64_t b_stride_n,
              int64_t out_stride_m, int64_t out_stride_n,
-             int32_t in_dtype, int32_t out_dtype, void* stream);
+             int32_t in_dtype, int32_t out_dtype,
+             void* workspace, int64_t workspace_bytes, void* stream);
 
 /* 2D x 3D with the rows of the first operand gathered on the fly:
  *   out[r, :] = a[row_index[r], :] @ b[g(r)]   for r < offs[G-1], g(r) the group that owns row r.
@@ -70,7 +90,8 @@ int gmm_2d3d_gather(const void* a, const int32_t* row_index, const void* b, void
                     int64_t a_stride_m, int64_t a_stride_k,
                     int64_t b_stride_g, int64_t b_stride_k, int64_t b_stride_n,
                     int64_t out_stride_m, int64_t out_stride_n,
-                    int32_t in_dtype, int32_t out_dtype, void* stream);
+                    int32_t in_dtype, int32_t out_dtype,
+                    void* workspace, int64_t workspace_bytes, void* stream);
 
 /* 2D x 3D with the SwiGLU activation applied to the product before it is stored (and, optionally, the row
  * gather above: row_index may be NULL for rows already in place, a_rows is then ignored).
@@ -96,7 +117,8 @@ int gmm_3d3d(const void* a, const void* b, void* out, int32_t G,
              int64_t a_stride_g, int64_t a_stride_m, int64_t a_stride_k,
              int64_t b_stride_g, int64_t b_stride_k, int64_t b_stride_n,
              int64_t out_stride_g, int64_t out_stride_m, int64_t out_stride_n,
-             int32_t in_dtype, int32_t out_dtype, void* stream);
+             int32_t in_dtype, int32_t out_dtype,
+             void* workspace, int64_t workspace_bytes, void* stream);
 
 /* 2D x 2D: out[g] = a[:, s_g:e_g] @ b[s_g:e_g, :]   (contraction jagged; zeros if empty)
  * a [M, K_total], b [K_total, N], out [G, M, N].
@@ -106,7 +128,8 @@ int gmm_2d2d(const void* a, const void* b, void* out, const int32_t* offs, int32
              int64_t a_stride_m, int64_t a_stride_k,
              int64_t b_stride_k, int64_t b_stride_n,
              int64_t out_stride_g, int64_t out_stride_m, int64_t out_stride_n,
-             int32_t in_dtype, int32_t out_dtype, void* stream);
+             int32_t in_dtype, int32_t out_dtype,
+             void* workspace, int64_t workspace_bytes, void* stream);
 
 /* 3D x 2D: out[:, s_g:e_g] = a[g] @ b[:, s_g:e_g]   (columns jagged)
  * a [G, M, K], b [K, N_total], out [M, N_total].
@@ -116,7 +139,8 @@ int gmm_3d2d(const void* a, const void* b, void* out, const int32_t* offs, int32
              int64_t a_stride_g, int64_t a_stride_m, int64_t a_stride_k,
              int64_t b_stride_k, int64_t b_stride_n,
              int64_t out_stride_m, int64_t out_stride_n,
-             int32_t in_dtype, int32_t out_dtype, void* stream);
+             int32_t in_dtype, int32_t out_dtype,
+             void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- The mixture-of-experts step either side of the grouped product.  The reference has no such code;
  * its benchmark builds the sorted rows and `offs` with torch on the host side (bench/bench_2d3d.py:124-149:
@@ -182,6 +206,13 @@ int gmm_set_mfma_config(int config);
 int gmm_last_mfma_config(void);
 /* 0 / 1: renumber tiles per XCD (default 1). */
 int gmm_set_xcd_remap(int on);
+/* Launch order of the assembly tile's kernel: 0 = all tall tiles of all groups, then the remainder tiles;
+ * 1 = group by group; -1 (default) = chosen from the shapes (group by group when the tall tiles are 128 rows,
+ * the regime of many small groups).  Returns the previous setting. */
+int gmm_set_group_major(int mode);
+/* 0: later launches ignore their workspace, so no tile is cut along the contraction (tests compare launches
+ * bit for bit that would otherwise split differently); 1 (default): use it.  Returns the previous setting. */
+int gmm_set_tail_split(int on);
 /* Tile heights of the assembly tile: tall = 256 or 128 (-1: chosen from the shapes), shrt = 64 or 0
  * (-1: 64 whenever the first operand is contiguous along the contraction).  Returns the previous
  * setting packed as ((tall + 1) << 16) | (shrt + 1). */
@@ -205,6 +236,17 @@ int64_t gmm_host_tile_list2(const int32_t* offs_host, int32_t G, int32_t jagged,
                             int32_t tall, int32_t shrt, int32_t tile_n, int32_t align,
                             int32_t xcd_remap, int32_t num_workgroups,
                             int32_t* records, int64_t capacity);
+
+/* The same list as a launch with a workspace of `max_parts` slots runs it: the tiles of the last, partly
+ * filled round cut along the contraction (see gmm_workspace_bytes), listed after the others in the order in
+ * which free workgroups draw them.  group_major != 0: the launch order is group by group (a group's tall
+ * tiles, then its remainder tiles) instead of all tall tiles first.  Records of 12 int32: the ten above
+ * (k_lo / k_hi are the part's range), the part's index and the number of parts of its tile (1: not split). */
+int64_t gmm_host_tile_list3(const int32_t* offs_host, int32_t G, int32_t jagged,
+                            int32_t M, int32_t N, int32_t K,
+                            int32_t tall, int32_t shrt, int32_t tile_n, int32_t align,
+                            int32_t xcd_remap, int32_t num_workgroups, int32_t max_parts,
+                            int32_t group_major, int32_t* records, int64_t capacity);
 
 /* Diagnostic, no counterpart in the reference: launches a register-only loop of independent
  * v_mfma_f32_32x32x16_bf16 on every SIMD (waves_per_simd 1 or 2; 16 MFMAs of 32768 FLOP per wave and

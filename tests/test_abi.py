@@ -21,7 +21,7 @@ def declared_functions():
 def test_library_exists_and_loads():
     assert os.path.exists(_lib.LIB_PATH), "build with: python -m grouped_mm_bf16_amd.build"
     lib = _lib.load()
-    assert lib.gmm_abi_version() == _lib.ABI_VERSION == 2
+    assert lib.gmm_abi_version() == _lib.ABI_VERSION == 3
 
 
 def test_every_declared_symbol_is_exported_and_bound():

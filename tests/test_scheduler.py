@@ -218,3 +218,117 @@ def test_two_heights_fine_grained_fixture(golden_dir):
     assert (coverage2(rec, 128, 32768, 768, False) == 1).all()
     rows_paid = sum(int(r[9]) for r in rec if r[2] == 0)
     assert rows_paid < 1.2 * 32768  # 256-row tiles alone pay for 54784 rows here
+
+
+# ---------------------------------------------------------------- last round cut along K (split workspace)
+def tile_list3(sizes, jag, M, N, K, tall, shrt, max_parts, align=1, remap=1, num_wg=256, group_major=0):
+    lib = _lib.load()
+    offs = np.cumsum(sizes).astype(np.int32) if jag != NONE else np.zeros(1, np.int32)
+    G = len(sizes)
+    n = lib.gmm_host_tile_list3(offs.ctypes.data, G, jag, M, N, K, tall, shrt, 256, align, remap, num_wg, max_parts, group_major, None, 0)
+    assert n >= 0
+    rec = np.zeros((max(n, 1), 12), np.int32)
+    assert lib.gmm_host_tile_list3(offs.ctypes.data, G, jag, M, N, K, tall, shrt, 256, align, remap, num_wg, max_parts,
+                                   group_major, rec.ctypes.data, n) == n
+    return rec[:n]
+
+
+def k_coverage(rec, K):
+    """Per output tile (group, m0, n0, rows): the K ranges of its records must partition [0, K) in part order."""
+    by_tile = {}
+    for r in rec:
+        by_tile.setdefault((int(r[0]), int(r[1]), int(r[2]), int(r[9])), []).append((int(r[10]), int(r[7]), int(r[8]), int(r[11])))
+    n_split = 0
+    for key, parts in by_tile.items():
+        parts.sort()
+        assert [p[0] for p in parts] == list(range(len(parts))), key
+        assert all(p[3] == len(parts) for p in parts), key
+        assert parts[0][1] == 0 and parts[-1][2] == K, key
+        for (_, _, hi, _), (_, lo, _, _) in zip(parts, parts[1:]):
+            assert hi == lo and lo % 64 == 0
+        assert all(hi - lo >= 24 * 64 or len(parts) == 1 for _, lo, hi, _ in parts)
+        n_split += len(parts) > 1
+    return by_tile, n_split
+
+
+MIXTRAL = [4812, 1663, 1610, 1663, 1656, 1682, 1633, 1665]
+
+
+def test_down_projection_tail_is_cut_five_ways():
+    """16384 x 14336 -> 4096 on 256 workgroups: 1008 tall + 80 remainder tiles = 4 rounds + 64 tiles; the 64
+    tiles of the fifth round become 320 parts of 44 or 45 K tiles each."""
+    whole = tile_list3(MIXTRAL, ROWS, 16384, 4096, 14336, 256, 64, 0)
+    assert len(whole) == 1088 and (whole[:, 11] == 1).all()
+    rec = tile_list3(MIXTRAL, ROWS, 16384, 4096, 14336, 256, 64, 512)
+    assert len(rec) == 1024 + 5 * 64
+    by_tile, n_split = k_coverage(rec, 14336)
+    assert len(by_tile) == 1088 and n_split == 64
+    assert (rec[:1024, 11] == 1).all() and (rec[1024:, 11] == 5).all()
+    # without the K ranges the list is the unsplit one: same tiles, same owners
+    assert (coverage2(whole[:, :10], 8, 16384, 4096, False) == 1).all()
+    first_parts = rec[rec[:, 10] == 0][:, :10]
+    assert (coverage2(first_parts, 8, 16384, 4096, False) == 1).all()
+    # the parts come in ticket order: K part 0 of every tile of the round, then K part 1, ...
+    assert (rec[1024:, 10] == np.repeat(np.arange(5), 64)).all()
+    # a workspace too small for five parts per tile allows fewer
+    rec = tile_list3(MIXTRAL, ROWS, 16384, 4096, 14336, 256, 64, 128)
+    assert len(rec) == 1024 + 2 * 64
+
+
+def test_up_projection_is_left_alone():
+    """16384 x 4096 -> 14336: the last round holds 224 of 256 tiles; cutting them would cost more than it saves."""
+    rec = tile_list3(MIXTRAL, ROWS, 16384, 14336, 4096, 256, 64, 512)
+    assert len(rec) == 3808 and (rec[:, 11] == 1).all()
+
+
+@pytest.mark.parametrize("jag,sizes,M,N", [(ROWS, [300, 0, 1, 255, 256, 257, 33], 1102, 700), (COLS, [129, 128, 127, 700], 330, 1084),
+                                           (NONE, [0] * 3, 330, 300)])
+@pytest.mark.parametrize("K", [1024, 1096, 4096, 16384])
+@pytest.mark.parametrize("num_wg,max_parts", [(256, 512), (64, 128), (16, 32), (8, 5)])
+def test_split_lists_cover_every_element_and_every_k(jag, sizes, M, N, K, num_wg, max_parts):
+    rec = tile_list3(sizes, jag, M, N, K, 256, 64, max_parts, align=8 if jag == COLS else 1, num_wg=num_wg)
+    by_tile, _ = k_coverage(rec, K)
+    first_parts = rec[rec[:, 10] == 0][:, :10]
+    G = len(sizes)
+    assert (coverage2(first_parts, G, M, N, jag == NONE) == 1).all()
+    unsplit = tile_list2(sizes, jag, M, N, K, 256, 64, align=8 if jag == COLS else 1, remap=1, num_wg=num_wg)
+    assert len(by_tile) == len(unsplit)
+    nparts = set(int(r[11]) for r in rec)
+    assert len(nparts - {1}) <= 1 and max(nparts) <= 8
+    if max(nparts) > 1:
+        n_parts_total = int((rec[:, 11] > 1).sum())
+        assert n_parts_total <= max_parts and len(rec) == len(unsplit) + n_parts_total - n_parts_total // max(nparts)
+
+
+def test_contraction_jagged_lists_are_never_split():
+    rec = tile_list3([4000, 5000, 7384], CONTRACTION, 330, 300, 16384, 256, 64, 512)
+    assert (rec[:, 11] == 1).all()
+
+
+@pytest.mark.parametrize("sizes", SIZE_LISTS + [MIXTRAL, [129, 128, 127, 65, 64, 63, 1]])
+@pytest.mark.parametrize("tall,remap", [(256, 0), (128, 0), (128, 1)])
+def test_group_major_order_covers_the_same_tiles(sizes, tall, remap):
+    """Group by group: the same tiles as the tall-first order, every group's remainder tiles right after its
+    tall tiles, groups in order."""
+    M, N = sum(sizes), 600
+    if M == 0:
+        return
+    a = tile_list3(sizes, ROWS, M, N, 64, tall, 64, 0, remap=remap, num_wg=16, group_major=1)
+    b = tile_list3(sizes, ROWS, M, N, 64, tall, 64, 0, remap=remap, num_wg=16, group_major=0)
+    assert sorted(map(tuple, a.tolist())) == sorted(map(tuple, b.tolist()))
+    assert (coverage2(a[:, :10], len(sizes), M, N, False) == 1).all()
+    if not remap:
+        groups = [int(r[0]) for r in a]
+        assert groups == sorted(groups)
+        for g in set(groups):
+            hs = [int(r[9]) for r in a if r[0] == g]
+            assert hs == sorted(hs, reverse=True)
+
+
+def test_fine_grained_fixture_group_major_with_split(golden_dir):
+    import json, os
+    with open(os.path.join(golden_dir, "group_sizes.json")) as f:
+        sizes = json.load(f)["fine_grained_top8_g128"]
+    rec = tile_list3(sizes, ROWS, 32768, 768, 2048, 128, 64, 512, group_major=1)
+    assert (rec[:, 11] == 1).all()          # 32 K tiles: too short a contraction to cut
+    assert (coverage2(rec[:, :10], 128, 32768, 768, False) == 1).all()
