@@ -30,7 +30,8 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 SETTLE_S = 0.15            # seconds of untimed launches before warm-up, after the host-side parity check
 # workload -> tag in the name of its rocprofv3 summary under profiles/ (`..__<tag>.md`)
-PROFILE_TAG = {"readme": "readme_2d3d", "mixtral": "mixtral_2d3d", "fine": "fine_grained_2d3d", "batched": "batched_3d3d",
+PROFILE_TAG = {"readme": "readme_2d3d", "mixtral": "mixtral_2d3d", "mixtral_colmajor": "mixtral_colmajor_2d3d",
+               "downproj": "downproj_2d3d", "fine": "fine_grained_2d3d", "batched": "batched_3d3d",
                "batched_colmajor": "batched_colmajor_3d3d", "kgrouped": "kgrouped_2d2d", "ngrouped": "ngrouped_3d2d"}
 
 
@@ -67,14 +68,26 @@ def make_workload(name, torch):
                  flops=2.0 * 32 * 64 * 48, bound="latency", k=64,
                  bytes=a.numel() * 2 + 4 * 64 * 48 * 2 + 32 * 48 * 2,
                  desc="readme_2d3d_G6_M32_K64_N48_two_empty_groups")
-    elif name == "mixtral":
+    elif name in ("mixtral", "mixtral_colmajor"):
+        # mixtral_colmajor: the weights as a linear layer stores them, [G, N, K] viewed transposed
         sizes = load_sizes("mixtral_top2_g8")
         a = torch.randn(16384, 4096, generator=g1).to(bf)
         b = (torch.randn(8, 4096, 14336, generator=g2) * 0.02).to(bf)
         w = dict(variant="2d3d", sizes=sizes, a=a, b=b, out_shape=(16384, 14336), out_dtype=bf,
                  flops=2.0 * 16384 * 4096 * 14336, bound="mfma", k=4096,
                  bytes=a.numel() * 2 + b.numel() * 2 + 16384 * 14336 * 2,
-                 desc="mixtral_moe_up_proj_2d3d_G8_M16384_K4096_N14336_skewed_top2")
+                 desc="mixtral_moe_up_proj_2d3d_G8_M16384_K4096_N14336_skewed_top2" + ("_Bcolmajor" if name.endswith("colmajor") else ""),
+                 b_col=name.endswith("colmajor"))
+    elif name == "downproj":
+        # the down projection of the same layer (and the input gradient of the up projection): the same FLOPs
+        # with a 3.5 times longer contraction and 4.25 rounds of tiles on 256 compute units
+        sizes = load_sizes("mixtral_top2_g8")
+        a = torch.randn(16384, 14336, generator=g1).to(bf)
+        b = (torch.randn(8, 14336, 4096, generator=g2) * 0.02).to(bf)
+        w = dict(variant="2d3d", sizes=sizes, a=a, b=b, out_shape=(16384, 4096), out_dtype=bf,
+                 flops=2.0 * 16384 * 14336 * 4096, bound="mfma", k=14336,
+                 bytes=a.numel() * 2 + b.numel() * 2 + 16384 * 4096 * 2,
+                 desc="mixtral_moe_down_proj_2d3d_G8_M16384_K14336_N4096_skewed_top2")
     elif name == "fine":
         sizes = load_sizes("fine_grained_top8_g128")
         a = torch.randn(32768, 2048, generator=g1).to(bf)
@@ -434,9 +447,17 @@ def run_moe(name, steps, warmup, torch, dev):
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
     flops = 2 * T * k * H * 2 * I + 2 * T * k * I * H
+    # algorithmic bytes of the layer: its inputs once (tokens, logits, both weight slabs of every expert that
+    # has a token) and its output once; what the stages hand to each other is the implementation's own traffic
+    offs = moe.moe_route(logits, k).offs.cpu()
+    used = int((torch.diff(offs, prepend=torch.zeros(1, dtype=offs.dtype)) > 0).sum())
+    nbytes = T * H * 2 + T * E * 4 + used * (H * 2 * I + I * H) * 2 + T * H * 2
+    tflops, gbs = flops / (ms * 1e-3) / 1e12, nbytes / (ms * 1e-3) / 1e9
+    hbm_bound = nbytes / PEAK_HBM_GBS > flops / (PEAK_BF16_TFLOPS * 1e3)     # which floor is the higher one
     return {"workload": f"MoE layer: {T} tokens, hidden {H}, inner {I} (SwiGLU in the up projection's epilogue), {E} experts, top {k}, bf16",
-            "ms": round(ms, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 2), "bound": "mfma" if name == "moe_mixtral" else "hbm",
-            "frac": round(flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4) if name == "moe_mixtral" else None,
+            "ms": round(ms, 4), "tflops": round(tflops, 2), "gbs": round(gbs, 1), "bound": "hbm" if hbm_bound else "mfma",
+            "frac": round(gbs / PEAK_HBM_GBS if hbm_bound else tflops / PEAK_BF16_TFLOPS, 4),
+            "algorithmic_flops": flops, "algorithmic_bytes": nbytes, "experts_with_tokens": used,
             "parity": "ok", "steps": steps}
 
 
@@ -446,7 +467,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="mixtral",
-                    choices=["mixtral", "readme", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "plain",
+                    choices=["mixtral", "mixtral_colmajor", "downproj", "readme", "fine", "batched", "batched_colmajor", "kgrouped", "ngrouped", "plain",
                              "copy", "mfma_only", "moe_mixtral", "moe_fine"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true",
@@ -516,7 +537,7 @@ def main():
         # The other benchmark configurations, a few steps each (kernel time from HIP events; the headline
         # fields above are the Mixtral workload's alone).
         rec["configs"] = {}
-        for name in ("readme", "batched", "batched_colmajor", "fine", "kgrouped"):
+        for name in ("readme", "mixtral_colmajor", "downproj", "batched", "batched_colmajor", "fine", "kgrouped", "ngrouped"):
             try:
                 wi, ri = run_workload(name, 30, 10, torch, dev, args.path, wall=False, settle_s=0.15)
                 k_avg = ri["roofline"]["kernel_ms_avg"]

@@ -121,14 +121,17 @@ __global__ void __launch_bounds__(256) moe_topk_kernel(const T* __restrict__ log
     if (lane == j) { my_e = e_win; my_key = key_win; }
     if (j == 0) top_key = key_win;
   }
+  // exp(x - m) with an infinite maximum m (a +inf logit, or a row of -inf: every expert masked) is the limit
+  // of the softmax: all weight, in equal shares, on the entries that equal the maximum (inf - inf is NaN)
   const float m = key_value(top_key);
-  const float p = lane < k ? __expf(key_value(my_key) - m) : 0.0f;
+  const bool inf_max = (__float_as_uint(m) & 0x7fffffffu) == 0x7f800000u;
+  const float p = lane < k ? (inf_max ? (my_key == top_key ? 1.0f : 0.0f) : __expf(key_value(my_key) - m)) : 0.0f;
   float den;
   if (renorm) {
     den = wave_sum(p);
   } else {
     float s = 0.0f;
-    for (int e = lane; e < E; e += 64) s += __expf(key_value(kw[e]) - m);
+    for (int e = lane; e < E; e += 64) s += inf_max ? (kw[e] == top_key ? 1.0f : 0.0f) : __expf(key_value(kw[e]) - m);
     den = wave_sum(s);
   }
   if (lane < k) {

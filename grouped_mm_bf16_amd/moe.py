@@ -74,6 +74,15 @@ def moe_route(router_logits: torch.Tensor, top_k: int, renormalize: bool = True)
     return r
 
 
+def _check_out(out: torch.Tensor, shape, like: torch.Tensor, what: str) -> None:
+    """A caller-supplied output must be exactly what the call computes: the kernels write through a raw pointer."""
+    if tuple(out.shape) != tuple(shape) or out.dtype != like.dtype or out.device != like.device:
+        raise RuntimeError(f"{what}: out has to be {tuple(shape)} {like.dtype} on {like.device}, "
+                           f"got {tuple(out.shape)} {out.dtype} on {out.device}")
+    if out.dim() != 2 or (out.numel() and (out.stride(1) != 1 or out.stride(0) < out.size(1))):
+        raise RuntimeError(f"{what}: out has to be row-major, got strides {tuple(out.stride())}")
+
+
 def grouped_mm_gathered(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tensor, offs: torch.Tensor,
                         out: torch.Tensor | None = None) -> torch.Tensor:
     """``grouped_mm(a[row_index], b, offs=offs)`` without materialising ``a[row_index]``.
@@ -90,13 +99,15 @@ def grouped_mm_gathered(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tenso
         raise RuntimeError("contraction dimension of mat_a and mat_b must match")
     if row_index.dtype != torch.int32 or row_index.dim() != 1 or not row_index.is_contiguous():
         raise RuntimeError("row_index has to be a contiguous 1D int32 tensor")
-    if offs.dtype != torch.int32 or offs.dim() != 1:
+    if offs.dtype != torch.int32 or offs.dim() != 1 or not offs.is_contiguous():
         raise RuntimeError("Offsets have to be int32")
     if offs.numel() != b.size(0):
         raise RuntimeError("matrix batch sizes have to match")
     M, N = row_index.numel(), b.size(2)
     if out is None:
         out = torch.empty(M, N, device=a.device, dtype=a.dtype)
+    else:
+        _check_out(out, (M, N), a, "grouped_mm_gathered")
     if M == 0 or N == 0:
         return out
     if a.size(1) == 0:
@@ -136,12 +147,14 @@ def grouped_mm_swiglu(a: torch.Tensor, row_index: torch.Tensor | None, b: torch.
         raise RuntimeError("grouped_mm_swiglu takes a [R, K] and b [G, K, N] of one dtype")
     if row_index is not None and (row_index.dtype != torch.int32 or row_index.dim() != 1 or not row_index.is_contiguous()):
         raise RuntimeError("row_index has to be a contiguous 1D int32 tensor")
-    if offs.dtype != torch.int32 or offs.dim() != 1 or offs.numel() != b.size(0):
+    if offs.dtype != torch.int32 or offs.dim() != 1 or offs.numel() != b.size(0) or not offs.is_contiguous():
         raise RuntimeError("offs has to be int32 [G]")
     M = row_index.numel() if row_index is not None else a.size(0)
     N = b.size(2)
     if out is None:
         out = torch.empty(M, N // 2, device=a.device, dtype=a.dtype)
+    else:
+        _check_out(out, (M, N // 2), a, "grouped_mm_swiglu")
     lib = _lib.load()
     with _guard(a):
         rc = lib.gmm_2d3d_swiglu(a.data_ptr(), row_index.data_ptr() if row_index is not None else None, b.data_ptr(),
@@ -166,6 +179,8 @@ def moe_activation(h: torch.Tensor, kind: str = "swiglu", out: torch.Tensor | No
     inner = h.size(1) // 2 if code else h.size(1)
     if out is None:
         out = torch.empty(h.size(0), inner, device=h.device, dtype=h.dtype)
+    else:
+        _check_out(out, (h.size(0), inner), h, "moe_activation")
     lib = _lib.load()
     with _guard(h):
         rc = lib.gmm_moe_activation(h.data_ptr(), out.data_ptr(), h.size(0), inner, h.stride(0) if h.size(0) else inner,
@@ -181,8 +196,15 @@ def moe_combine(y: torch.Tensor, routing: Routing, tokens: int, top_k: int, out:
     if y.dim() != 2 or (y.numel() and y.stride(1) != 1):
         raise RuntimeError("moe_combine takes a row-major 2D tensor")
     H = y.size(1)
+    slots = tokens * top_k
+    for name, t, dt in (("token_rows", routing.token_rows, torch.int32), ("slot_weight", routing.slot_weight, torch.float32)):
+        if t.dtype != dt or t.numel() != slots or not t.is_contiguous() or t.device != y.device:
+            raise RuntimeError(f"moe_combine: routing.{name} has to be a contiguous {dt} tensor of tokens * top_k = {slots} "
+                               f"elements on {y.device}, got {t.numel()} of {t.dtype} on {t.device}")
     if out is None:
         out = torch.empty(tokens, H, device=y.device, dtype=y.dtype)
+    else:
+        _check_out(out, (tokens, H), y, "moe_combine")
     lib = _lib.load()
     with _guard(y):
         rc = lib.gmm_moe_combine(y.data_ptr(), routing.token_rows.data_ptr(), routing.slot_weight.data_ptr(), out.data_ptr(),

@@ -147,7 +147,9 @@ int gmm_3d2d(const void* a, const void* b, void* out, const int32_t* offs, int32
  * randint / bincount / cumsum and an offs[-1].item() round trip).  Here everything stays on the device.
  *
  * Routing.  For each of `tokens` rows of `logits` [tokens, experts] (row stride logits_stride elements,
- * dtype a gmm_dtype) pick the top_k largest (ties: lower expert index first; logits must not be NaN), in
+ * dtype a gmm_dtype) pick the top_k largest (ties: lower expert index first; logits must not be NaN; -inf
+ * masks an expert; a row whose maximum is +inf or -inf puts all weight, in equal shares, on the entries equal
+ * to the maximum: the limit of the softmax), in
  * descending order.  Choice j of token t is SLOT t * top_k + j.  Outputs (device memory):
  *   slot_expert int32[tokens * top_k]   expert of each slot
  *   slot_weight float[tokens * top_k]   softmax over the token's chosen logits (renormalize != 0), or the
@@ -172,7 +174,10 @@ int gmm_moe_route(const void* logits, int64_t logits_stride, int32_t logits_dtyp
  * gmm_moe_route_workspace_bytes(...) exceeds 262144 bytes are refused with GMM_ERR_WORKSPACE (any problem
  * with experts <= 256 fits; with 1023 experts up to 65536 slots).  All calls on one GPU share that array:
  * calls that may overlap on one GPU (different streams, different threads) race and must be serialised by
- * the caller.  Outputs and everything else as gmm_moe_route. */
+ * the caller.  The first call on a device looks the array's device address up (hipGetSymbolAddress, no
+ * allocation): make that first call outside a stream capture -- one eager call per device at start-up is
+ * enough -- and every later call, captured or not, only launches.  Outputs and everything else as
+ * gmm_moe_route. */
 int gmm_moe_route_noalloc(const void* logits, int64_t logits_stride, int32_t logits_dtype,
                           int64_t tokens, int64_t experts, int64_t top_k, int32_t renormalize,
                           int32_t* offs, int32_t* slot_expert, float* slot_weight,

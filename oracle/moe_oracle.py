@@ -43,6 +43,11 @@ def route(logits: torch.Tensor, top_k: int, renormalize: bool = True) -> Routing
     order = torch.sort(lf, dim=-1, descending=True, stable=True)
     chosen = order.indices[:, :top_k]                                   # [T, k], descending, ties -> lower index
     probs = torch.softmax(lf, dim=-1)
+    # a row whose maximum is infinite (a +inf logit, or every logit -inf): the softmax's limit, all weight in
+    # equal shares on the entries that equal the maximum (torch.softmax itself returns NaN there)
+    top = lf.max(dim=-1, keepdim=True).values
+    at_top = (lf == top).float()
+    probs = torch.where(torch.isinf(top), at_top / at_top.sum(dim=-1, keepdim=True), probs)
     w = torch.gather(probs, 1, chosen)
     if renormalize:
         w = w / w.sum(dim=-1, keepdim=True)

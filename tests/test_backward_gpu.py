@@ -213,8 +213,6 @@ ALIGNED = {  # variant -> (sizes along the jagged dimension, d1, d2): every exte
 def test_backward_on_the_assembly_tile(variant, layout, dtype):
     """bf16 / fp16 with aligned extents: the forward and both gradient launches take the MFMA family (the
     gradients through transposed views, with jagged contractions starting at odd k)."""
-    if dtype == torch.float16 and layout != (False, False):
-        pytest.skip("fp16 shares every layout path with bf16; one layout is enough")
     gen = torch.Generator().manual_seed(5)
     sizes, d1, d2 = ALIGNED[variant]
     extra = 0 if variant == "3d3d" else 8 - sum(sizes) % 8   # pad the jagged extent to a multiple of 8

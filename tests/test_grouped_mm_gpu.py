@@ -296,15 +296,16 @@ def test_tile_heights_agree_bit_for_bit(tall, shrt, b_col):
 
 @pytest.mark.parametrize("a_col", [False, True])
 @pytest.mark.parametrize("b_col", [False, True])
-@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("in_dtype,out_dtype", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                               (torch.float16, torch.float16), (torch.float16, torch.float32)])
 @pytest.mark.parametrize("sizes", [[77, 0, 1, 330, 64, 200], [8, 16, 256, 512, 24], [3, 5, 7, 9, 300, 1, 600]])
-def test_3d2d_on_the_assembly_tile(sizes, out_dtype, a_col, b_col):
+def test_3d2d_on_the_assembly_tile(sizes, in_dtype, out_dtype, a_col, b_col):
     """Jagged columns: group boundaries inside a 16-byte chunk of the output go out as element stores;
     nothing outside a group's columns (and nothing past the last offset) is written."""
     gen = torch.Generator().manual_seed(31 + len(sizes))
     G, n_total = len(sizes), sum(sizes)
     extra = 16 + (-n_total % 8)   # columns past the last offset belong to nobody; the total is a multiple of 8
-    a, b = rnd(gen, G, 328, 200), rnd(gen, 200, n_total + extra, scale=0.05)
+    a, b = rnd(gen, G, 328, 200, dtype=in_dtype), rnd(gen, 200, n_total + extra, scale=0.05, dtype=in_dtype)
     offs = offs_of(sizes)
     ad, bd = a.to(DEV), b.to(DEV)
     if a_col:
@@ -703,13 +704,36 @@ def test_mixtral_up_projection_full_size(golden_dir):
     oracle.assert_close(out[4700:4900].cpu(), ref_band.cpu(), 4096)
 
 
-def test_fine_grained_moe_full_size(golden_dir):
+def test_mixtral_up_projection_full_size_column_major_weights(golden_dir):
+    """The weights as a linear layer stores them, [G, N, K] viewed transposed (B contiguous along K): whole
+    output against the oracle, and the same bits as the row-major launch (same K order)."""
+    sizes = _sizes(golden_dir, "mixtral_top2_g8")
+    offs = offs_of(sizes)
+    a = rnd(torch.Generator().manual_seed(1), 16384, 4096)
+    b = rnd(torch.Generator().manual_seed(2), 8, 4096, 14336, scale=0.02)
+    ad, bd = a.to(DEV), b.to(DEV)
+    b_nk = bd.transpose(1, 2).contiguous()           # [8, 14336, 4096]
+    out = torch.full((16384, 14336), float("nan"), device=DEV, dtype=torch.bfloat16)
+    K_.grouped_mm_2d3d(ad, b_nk.transpose(1, 2), offs.to(DEV), out)
+    assert K_.last_path() == "mfma" and K_._lib.load().gmm_last_mfma_config() == 1
+    assert not torch.isnan(out.float()).any()
+    _full_check_2d3d(out, a, b, offs.tolist(), 4096)
+    ref = torch.empty_like(out)
+    K_.grouped_mm_2d3d(ad, bd, offs.to(DEV), ref)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("b_col", [False, True])
+def test_fine_grained_moe_full_size(golden_dir, b_col):
     sizes = _sizes(golden_dir, "fine_grained_top8_g128")
     offs = offs_of(sizes)
     a = rnd(torch.Generator().manual_seed(1), 32768, 2048)
     b = rnd(torch.Generator().manual_seed(2), 128, 2048, 768, scale=0.02)
+    bd = b.to(DEV)
+    if b_col:
+        bd = bd.transpose(1, 2).contiguous().transpose(1, 2)
     out = torch.full((32768, 768), float("nan"), device=DEV, dtype=torch.bfloat16)
-    K_.grouped_mm_2d3d(a.to(DEV), b.to(DEV), offs.to(DEV), out)
+    K_.grouped_mm_2d3d(a.to(DEV), bd, offs.to(DEV), out)
     assert K_.last_path() == "mfma"
     want = oracle.grouped_mm(a, b, offs)  # 0.1 TFLOP: a few seconds on the host
     assert not torch.isnan(out.float()).any()

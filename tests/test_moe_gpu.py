@@ -64,6 +64,27 @@ def test_routing_fp16_skewed_padded_and_empty():
     assert r.offs.tolist() == [0] * 8 and r.slot_expert.numel() == 0
 
 
+@pytest.mark.parametrize("renorm", [True, False])
+def test_routing_with_infinite_logits(renorm):
+    """-inf masks an expert (weight exactly 0 if it is still chosen); a +inf logit takes all the weight, several
+    share it equally; a fully masked row spreads its weight over its choices (renormalised) or over all experts."""
+    gen = torch.Generator().manual_seed(21)
+    logits = torch.randn(64, 16, generator=gen)
+    logits[:, 5:11] = float("-inf")             # masked experts, never among the top 4 of 10 finite ones
+    logits[3, :] = float("-inf")                # every expert masked
+    logits[4, :14] = float("-inf")              # two finite logits, top_k = 4: two choices are masked experts
+    logits[7, 2] = float("inf")
+    logits[9, 1] = logits[9, 12] = float("inf")
+    got = moe.moe_route(logits.to(DEV), 4, renormalize=renorm)
+    want = moe_oracle.route(logits, 4, renorm)
+    check_routing(got, want)
+    w = got.slot_weight.cpu().view(64, 4)
+    assert torch.isfinite(w).all()
+    assert w[7].tolist() == [1.0, 0.0, 0.0, 0.0] and w[9].tolist() == [0.5, 0.5, 0.0, 0.0]
+    assert w[4, 2:].tolist() == [0.0, 0.0]
+    assert w[3].tolist() == ([0.25] * 4 if renorm else [1.0 / 16] * 4)
+
+
 def test_routing_rejects_what_it_cannot_do():
     lg = torch.zeros(4, 8, device=DEV)
     with pytest.raises(RuntimeError):

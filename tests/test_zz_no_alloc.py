@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from grouped_mm_bf16_amd import _lib
+from oracle import moe_oracle
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -41,6 +42,11 @@ def test_two_calls_in_a_row_match_the_workspace_entry_point():
         for name, g, w in zip(("offs", "slot_expert", "slot_weight", "row_token", "token_rows"), got, want):
             assert torch.equal(g, w), name
         assert int(got[0][-1]) == T * k and sorted(got[4].tolist()) == list(range(T * k))
+        # and against the oracle, so that a mistake both entry points share does not pass
+        ref = moe_oracle.route(logits.cpu(), k, bool(renorm))
+        assert torch.equal(got[0].cpu(), ref.offs) and torch.equal(got[1].cpu(), ref.slot_expert)
+        assert torch.equal(got[3].cpu(), ref.row_token) and torch.equal(got[4].cpu(), ref.token_rows)
+        torch.testing.assert_close(got[2].cpu(), ref.slot_weight, rtol=2e-5, atol=1e-7)
 
 
 def test_sizes_beyond_the_built_in_table_are_refused():
