@@ -8,7 +8,9 @@ and gets ``offs`` from ``bincount(...).cumsum(0)`` with a host round trip (``ben
 Here no count ever reaches the host: the kernels read ``offs`` from device memory, and every buffer is sized
 by ``tokens * top_k``, which the host knows.
 
-Forward only (inference); the functions take and return plain tensors.
+Forward only (inference); the functions take and return plain tensors.  Each one is also registered as a
+torch custom op (``grouped_mm_bf16_amd::moe_route``, ``gathered``, ``swiglu``, ``activation``, ``combine``) and
+dispatches to it while a model around it is being traced or compiled.
 """
 from __future__ import annotations
 
@@ -36,13 +38,9 @@ def _guard(t: torch.Tensor):
     return torch.cuda.device(t.device) if t.device.index != torch.cuda.current_device() else contextlib.nullcontext()
 
 
-def moe_route(router_logits: torch.Tensor, top_k: int, renormalize: bool = True) -> Routing:
-    """Top-k routing and the stable sort of the slots by expert.
-
-    router_logits [T, E] (bf16, fp16 or fp32, last dimension contiguous).  Ties go to the lower expert index;
-    weights are the softmax over the chosen logits (``renormalize``) or the chosen entries of the softmax
-    over all experts.
-    """
+def _route_packed_now(router_logits: torch.Tensor, top_k: int, renormalize: bool) -> torch.Tensor:
+    """The five routing results in one int32 buffer [E + 4 S] (offs, slot_expert, slot_weight bits, row_token,
+    token_rows): one allocation for results and workspace (each allocation costs microseconds of host time)."""
     _require_gpu(router_logits)
     if router_logits.dim() != 2:
         raise RuntimeError("router_logits has to be 2D [tokens, experts]")
@@ -58,20 +56,38 @@ def moe_route(router_logits: torch.Tensor, top_k: int, renormalize: bool = True)
     ws_bytes = lib.gmm_moe_route_workspace_bytes(T, E, top_k)
     if ws_bytes < 0:
         raise RuntimeError("moe_route: sizes out of range")
-    # one allocation for the five results and the workspace (each allocation costs microseconds of host time)
     buf = torch.empty(E + 4 * S + ws_bytes // 4, device=dev, dtype=torch.int32)
-    cut = [E, S, S, S, S]
-    parts = torch.split(buf[:E + 4 * S], cut)
-    r = Routing(parts[0], parts[1], parts[2].view(torch.float32), parts[3], parts[4])
-    ws = buf[E + 4 * S:]
+    base, ws = buf.data_ptr(), buf[E + 4 * S:]
     with _guard(router_logits):
         rc = lib.gmm_moe_route(router_logits.data_ptr(), router_logits.stride(0) if T else E,
                                _dtype_code(router_logits.dtype), T, E, top_k, int(bool(renormalize)),
-                               r.offs.data_ptr(), r.slot_expert.data_ptr(), r.slot_weight.data_ptr(),
-                               r.row_token.data_ptr(), r.token_rows.data_ptr(), ws.data_ptr(), ws_bytes,
-                               torch.cuda.current_stream().cuda_stream)
+                               base, base + 4 * E, base + 4 * (E + S), base + 4 * (E + 2 * S), base + 4 * (E + 3 * S),
+                               ws.data_ptr(), ws_bytes, torch.cuda.current_stream().cuda_stream)
     _lib.check(rc, "moe_route")
-    return r
+    return buf[:E + 4 * S]
+
+
+_route_op = torch.library.custom_op("grouped_mm_bf16_amd::moe_route", mutates_args=())(_route_packed_now)
+
+
+@_route_op.register_fake
+def _route_fake(router_logits, top_k, renormalize):
+    T, E = router_logits.shape
+    return router_logits.new_empty(E + 4 * T * top_k, dtype=torch.int32)
+
+
+def moe_route(router_logits: torch.Tensor, top_k: int, renormalize: bool = True) -> Routing:
+    """Top-k routing and the stable sort of the slots by expert.
+
+    router_logits [T, E] (bf16, fp16 or fp32, last dimension contiguous).  Ties go to the lower expert index;
+    weights are the softmax over the chosen logits (``renormalize``) or the chosen entries of the softmax
+    over all experts.
+    """
+    impl = _route_op if torch.compiler.is_compiling() else _route_packed_now
+    buf = impl(router_logits, top_k, bool(renormalize))
+    E, S = router_logits.size(1), router_logits.size(0) * top_k
+    parts = torch.split(buf, [E, S, S, S, S])
+    return Routing(parts[0], parts[1], parts[2].view(torch.float32), parts[3], parts[4])
 
 
 def _check_out(out: torch.Tensor, shape, like: torch.Tensor, what: str) -> None:
@@ -83,6 +99,11 @@ def _check_out(out: torch.Tensor, shape, like: torch.Tensor, what: str) -> None:
         raise RuntimeError(f"{what}: out has to be row-major, got strides {tuple(out.stride())}")
 
 
+def _no_out_when_compiling(out, what: str) -> None:
+    if out is not None:
+        raise RuntimeError(f"{what}: out= is not available under torch.compile (the traced ops allocate their results)")
+
+
 def grouped_mm_gathered(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tensor, offs: torch.Tensor,
                         out: torch.Tensor | None = None) -> torch.Tensor:
     """``grouped_mm(a[row_index], b, offs=offs)`` without materialising ``a[row_index]``.
@@ -90,6 +111,14 @@ def grouped_mm_gathered(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tenso
     a [R_src, K], row_index int32 [M_total], b [G, K, N], offs int32 [G]; returns [M_total, N] in a's dtype.
     An index outside [0, R_src) reads a row of zeros.
     """
+    if torch.compiler.is_compiling():
+        _no_out_when_compiling(out, "grouped_mm_gathered")
+        return _gathered_op(a, row_index, b, offs)
+    return _gathered_now(a, row_index, b, offs, out)
+
+
+def _gathered_now(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tensor, offs: torch.Tensor,
+                  out: torch.Tensor | None = None) -> torch.Tensor:
     _require_gpu(a, row_index, b, offs)
     if a.dim() != 2 or b.dim() != 3:
         raise RuntimeError("grouped_mm_gathered takes a 2D first and a 3D second operand")
@@ -124,6 +153,20 @@ def grouped_mm_gathered(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tenso
     return out
 
 
+def _gathered_functional(a: torch.Tensor, row_index: torch.Tensor, b: torch.Tensor, offs: torch.Tensor) -> torch.Tensor:
+    return _gathered_now(a, row_index, b, offs)
+
+
+# The functions of this module as torch custom ops (functional: they allocate their result), for callers that
+# trace or compile a model around them.  Eager calls skip the dispatcher.
+_gathered_op = torch.library.custom_op("grouped_mm_bf16_amd::gathered", mutates_args=())(_gathered_functional)
+
+
+@_gathered_op.register_fake
+def _gathered_fake(a, row_index, b, offs):
+    return a.new_empty(row_index.numel(), b.size(2))
+
+
 def interleave_gate_up(w_up: torch.Tensor) -> torch.Tensor:
     """[E, H, 2I] with all gate columns first, then all partner ("up") columns  ->  the layout the fused SwiGLU
     epilogue wants: in every block of 128 columns, 64 gate columns followed by their 64 partners.  I must be a
@@ -142,6 +185,14 @@ def grouped_mm_swiglu(a: torch.Tensor, row_index: torch.Tensor | None, b: torch.
     """``swiglu(grouped_mm(a[row_index], b, offs))`` in one kernel, for ``b`` in the layout of
     :func:`interleave_gate_up`; the [M_total, N] intermediate is never written.  Returns [M_total, N / 2].
     Raises if the operands do not qualify for the fast path (see ``gmm_2d3d_swiglu`` in the C header)."""
+    if torch.compiler.is_compiling():
+        _no_out_when_compiling(out, "grouped_mm_swiglu")
+        return _swiglu_op(a, row_index, b, offs)
+    return _swiglu_now(a, row_index, b, offs, out)
+
+
+def _swiglu_now(a: torch.Tensor, row_index: torch.Tensor | None, b: torch.Tensor, offs: torch.Tensor,
+                out: torch.Tensor | None = None) -> torch.Tensor:
     _require_gpu(a, row_index, b, offs)
     if a.dim() != 2 or b.dim() != 3 or a.dtype != b.dtype or a.size(1) != b.size(1):
         raise RuntimeError("grouped_mm_swiglu takes a [R, K] and b [G, K, N] of one dtype")
@@ -165,9 +216,28 @@ def grouped_mm_swiglu(a: torch.Tensor, row_index: torch.Tensor | None, b: torch.
     return out
 
 
+def _swiglu_functional(a: torch.Tensor, row_index: torch.Tensor | None, b: torch.Tensor, offs: torch.Tensor) -> torch.Tensor:
+    return _swiglu_now(a, row_index, b, offs)
+
+
+_swiglu_op = torch.library.custom_op("grouped_mm_bf16_amd::swiglu", mutates_args=())(_swiglu_functional)
+
+
+@_swiglu_op.register_fake
+def _swiglu_fake(a, row_index, b, offs):
+    return a.new_empty(row_index.numel() if row_index is not None else a.size(0), b.size(2) // 2)
+
+
 def moe_activation(h: torch.Tensor, kind: str = "swiglu", out: torch.Tensor | None = None) -> torch.Tensor:
     """``silu(h)`` or, for "swiglu", ``silu(h[:, :I]) * h[:, I:]`` with I = h.size(1) // 2 (fp32 arithmetic,
     one rounding).  h [R, I or 2I], bf16 or fp16, row-major."""
+    if torch.compiler.is_compiling():
+        _no_out_when_compiling(out, "moe_activation")
+        return _activation_op(h, kind)
+    return _activation_now(h, kind, out)
+
+
+def _activation_now(h: torch.Tensor, kind: str = "swiglu", out: torch.Tensor | None = None) -> torch.Tensor:
     _require_gpu(h)
     if kind not in ACTIVATIONS:
         raise RuntimeError(f"unknown activation {kind!r}; have {sorted(ACTIVATIONS)}")
@@ -190,14 +260,34 @@ def moe_activation(h: torch.Tensor, kind: str = "swiglu", out: torch.Tensor | No
     return out
 
 
+def _activation_functional(h: torch.Tensor, kind: str) -> torch.Tensor:
+    return _activation_now(h, kind)
+
+
+_activation_op = torch.library.custom_op("grouped_mm_bf16_amd::activation", mutates_args=())(_activation_functional)
+
+
+@_activation_op.register_fake
+def _activation_fake(h, kind):
+    return h.new_empty(h.size(0), h.size(1) // 2 if ACTIVATIONS.get(kind) else h.size(1))
+
+
 def moe_combine(y: torch.Tensor, routing: Routing, tokens: int, top_k: int, out: torch.Tensor | None = None) -> torch.Tensor:
     """out[t] = sum_j slot_weight[t, j] * y[token_rows[t, j]] in fp32, rounded once.  y [S, H] row-major."""
+    if torch.compiler.is_compiling():
+        _no_out_when_compiling(out, "moe_combine")
+        return _combine_op(y, routing.token_rows, routing.slot_weight, tokens, top_k)
+    return _combine_now(y, routing.token_rows, routing.slot_weight, tokens, top_k, out)
+
+
+def _combine_now(y: torch.Tensor, token_rows: torch.Tensor, slot_weight: torch.Tensor, tokens: int, top_k: int,
+                 out: torch.Tensor | None = None) -> torch.Tensor:
     _require_gpu(y)
     if y.dim() != 2 or (y.numel() and y.stride(1) != 1):
         raise RuntimeError("moe_combine takes a row-major 2D tensor")
     H = y.size(1)
     slots = tokens * top_k
-    for name, t, dt in (("token_rows", routing.token_rows, torch.int32), ("slot_weight", routing.slot_weight, torch.float32)):
+    for name, t, dt in (("token_rows", token_rows, torch.int32), ("slot_weight", slot_weight, torch.float32)):
         if t.dtype != dt or t.numel() != slots or not t.is_contiguous() or t.device != y.device:
             raise RuntimeError(f"moe_combine: routing.{name} has to be a contiguous {dt} tensor of tokens * top_k = {slots} "
                                f"elements on {y.device}, got {t.numel()} of {t.dtype} on {t.device}")
@@ -207,11 +297,23 @@ def moe_combine(y: torch.Tensor, routing: Routing, tokens: int, top_k: int, out:
         _check_out(out, (tokens, H), y, "moe_combine")
     lib = _lib.load()
     with _guard(y):
-        rc = lib.gmm_moe_combine(y.data_ptr(), routing.token_rows.data_ptr(), routing.slot_weight.data_ptr(), out.data_ptr(),
+        rc = lib.gmm_moe_combine(y.data_ptr(), token_rows.data_ptr(), slot_weight.data_ptr(), out.data_ptr(),
                                  tokens, top_k, H, y.size(0), y.stride(0) if y.size(0) else H, out.stride(0) if tokens else H,
                                  _dtype_code(y.dtype), torch.cuda.current_stream().cuda_stream)
     _lib.check(rc, "moe_combine")
     return out
+
+
+def _combine_functional(y: torch.Tensor, token_rows: torch.Tensor, slot_weight: torch.Tensor, tokens: int, top_k: int) -> torch.Tensor:
+    return _combine_now(y, token_rows, slot_weight, tokens, top_k)
+
+
+_combine_op = torch.library.custom_op("grouped_mm_bf16_amd::combine", mutates_args=())(_combine_functional)
+
+
+@_combine_op.register_fake
+def _combine_fake(y, token_rows, slot_weight, tokens, top_k):
+    return y.new_empty(tokens, y.size(1))
 
 
 def moe_forward(x: torch.Tensor, router_logits: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, top_k: int,

@@ -413,3 +413,52 @@ def test_layer_replays_from_a_captured_graph():
         assert torch.equal(replayed.view(torch.int16), eager.view(torch.int16)), f"replay {rep} differs from eager"
         oracle.assert_close(replayed.cpu(), moe_oracle.moe_forward(x, logits, w_up, w_down, k, fused=True), I)
     assert len(seen) == 3, "the routing was meant to change between replays"
+
+
+# ------------------------------------------------------------------ the step as torch custom ops
+@pytest.mark.parametrize("fused", [False, True])
+def test_compiled_layer_goes_through_the_custom_ops(fused):
+    """torch.compile(fullgraph=True) of a function that calls moe_forward: every stage is reached through its
+    registered op (no graph break), and the compiled layer returns what the eager layer returns, bit for bit."""
+    T, H, I, E, k = 130, 136, 256, 6, 2
+    x, logits, w_up, w_down = layer_case(77, T, H, I, E, k, "swiglu")
+    wu = moe.interleave_gate_up(w_up.to(DEV)) if fused else w_up.to(DEV)
+    args = (x.to(DEV), logits.to(DEV), wu, w_down.to(DEV))
+
+    def layer(x_, lg_, wu_, wd_):
+        return moe.moe_forward(x_, lg_, wu_, wd_, k, "swiglu", True, interleaved=fused) * 2.0
+
+    eager = layer(*args)
+    torch._dynamo.reset()
+    compiled = torch.compile(layer, backend="aot_eager", fullgraph=True)(*args)
+    torch.cuda.synchronize()
+    assert torch.equal(eager.view(torch.int16), compiled.view(torch.int16))
+    want = moe_oracle.moe_forward(x, logits, w_up, w_down, k, "swiglu", True, fused=fused) * 2.0
+    oracle.assert_close(compiled.cpu(), want, I)
+
+
+def test_custom_ops_pass_opcheck_and_match_the_direct_calls():
+    T, H, I, E, k = 70, 136, 128, 5, 2
+    x, logits, w_up, w_down = layer_case(78, T, H, I, E, k, "swiglu")
+    xd, lg, wu = x.to(DEV), logits.to(DEV), w_up.to(DEV)
+    ops, checks = torch.ops.grouped_mm_bf16_amd, ("test_schema", "test_faketensor")
+    r = moe.moe_route(lg, k)
+    packed = ops.moe_route(lg, k, True)
+    assert torch.equal(packed[:E], r.offs) and torch.equal(packed[E + 2 * T * k:E + 3 * T * k], r.row_token)
+    torch.library.opcheck(ops.moe_route.default, (lg, k, True), test_utils=checks)
+    h = moe.grouped_mm_gathered(xd, r.row_token, wu, r.offs)
+    assert torch.equal(ops.gathered(xd, r.row_token, wu, r.offs).view(torch.int16), h.view(torch.int16))
+    torch.library.opcheck(ops.gathered.default, (xd, r.row_token, wu, r.offs), test_utils=checks)
+    wil = moe.interleave_gate_up(wu)
+    fused = moe.grouped_mm_swiglu(xd, r.row_token, wil, r.offs)
+    assert torch.equal(ops.swiglu(xd, r.row_token, wil, r.offs).view(torch.int16), fused.view(torch.int16))
+    torch.library.opcheck(ops.swiglu.default, (xd, r.row_token, wil, r.offs), test_utils=checks)
+    torch.library.opcheck(ops.swiglu.default, (fused, None, wil[:, :I], r.offs), test_utils=checks)
+    act = moe.moe_activation(h, "swiglu")
+    assert torch.equal(ops.activation(h, "swiglu").view(torch.int16), act.view(torch.int16))
+    torch.library.opcheck(ops.activation.default, (h, "silu"), test_utils=checks)
+    y = torch.empty(T * k, H, device=DEV, dtype=torch.bfloat16)
+    K_.grouped_mm_2d3d(act, w_down.to(DEV), r.offs, y)
+    out = moe.moe_combine(y, r, T, k)
+    assert torch.equal(ops.combine(y, r.token_rows, r.slot_weight, T, k).view(torch.int16), out.view(torch.int16))
+    torch.library.opcheck(ops.combine.default, (y, r.token_rows, r.slot_weight, T, k), test_utils=checks)
