@@ -12,8 +12,12 @@ the pipeline.  Here every register is named, so nothing is spilled and the issue
 order is exactly the one below.
 
 One block computes one 256 x 256 output tile with 4 waves (2 x 2, 128 x 128 per
-wave, 4 x 4 MFMA blocks of 32 x 32); variants for 128 x 256 and 64 x 256 tiles
-(group remainders, small groups) and for fp16 instead of bf16 elements:
+wave, 8 x 8 MFMA blocks of 16 x 16); variants for 128 x 256 and 64 x 256 tiles
+(group remainders, small groups) and for fp16 instead of bf16 elements.  The MFMA
+is v_mfma_f32_16x16x32: per FLOP it moves half the accumulator data of the
+32 x 32 x 16 shape through the register file, and in a register-only loop on
+operands drawn like the benchmark's it sustains 1960-2050 TFLOP/s where
+32 x 32 x 16 sustains 1790-1810 (the clock follows the power drawn):
 
   * K is walked in tiles of 64; A and B tiles are copied global -> LDS by
     buffer_load_dwordx4 ... lds (no registers involved) into two buffers (three
@@ -23,17 +27,22 @@ wave, 4 x 4 MFMA blocks of 32 x 32); variants for 128 x 256 and 64 x 256 tiles
     16-byte chunks XOR-swizzled (conflict-free ds_read_b128 fragments); one that
     is contiguous along M / N lives as [k][256] in blocks of two k rows with a
     64-byte pad, read with ds_read_b64_tr_b16 (the LDS transposes 4 x 16 blocks);
-  * per k16 step a wave issues 16 v_mfma_f32_32x32x16_bf16 and, between them, the
-    fragment reads of the next step (A block 0, the B blocks, then the other A
-    blocks: each MFMA waits only for its own operands, lgkmcnt counts down in
-    order) and its share of the copies of the next tiles;
+  * a K tile is four steps: (k 0..31, upper half of the wave's rows), (k 0..31,
+    lower half), (k 32..63, upper), (k 32..63, lower).  A step issues 8 tm
+    v_mfma_f32_16x16x32 (tm = 4 for the 256-row tile) and, between them, the
+    fragment reads the following steps need -- the A fragments of the next step
+    into the other of two A register sets, the B fragments of the next k half
+    into the other of two B sets -- and its share of the copies of the next
+    tiles.  LDS reads complete in order: every MFMA waits (lgkmcnt) only until
+    its own operands have arrived;
   * the loop body exists twice: K tiles whose copies are neither the last tile of
     the range nor past it use the copy offsets as they are; the others select
     per copy between the normal offsets, the last tile's offsets and "out of
     range" (a buffer load that fetches nothing and writes zeros);
   * one s_barrier per K tile, placed after step 2 so that step 3's MFMAs run
     while the barrier's stragglers arrive and the first fragments of the next
-    tile are fetched under them;
+    tile (its B fragments of k 0..31 and the A fragments of its step 0) are
+    fetched under them;
   * epilogue: the MFMA operands are swapped so a lane owns 4 consecutive columns;
     it packs them (v_cvt_pk_bf16_f32; fp32 goes as it is), stages the wave's block
     in LDS and writes 16 bytes per lane: 256 contiguous bytes per row (512 for
@@ -41,10 +50,11 @@ wave, 4 x 4 MFMA blocks of 32 x 32); variants for 128 x 256 and 64 x 256 tiles
     by element.
 
 Registers:
-  a[0:255]     accumulators, block (i, j) at a[(4 i + j) 16 ...]
-  v[0:15]      A fragments set 0, v[16:31] set 1, v[32:47] B set 0, v[48:63] B set 1
-  v[64:121]    temporaries, per-buffer fragment addresses of the 3-buffer variants
-  inputs are pinned by the C++ wrapper to v[128:...] and s[28:55] (see GmmTileRegs).
+  a[0:255]     accumulators, 16 x 16 block (i, j) at a[(8 i + j) 4 ...]
+  v[0:15]      A fragments set 0 (four of 16 rows x 32 k), v[16:31] set 1,
+  v[32:63]     B fragments set 0 (eight of 16 columns x 32 k), v[64:95] set 1
+  v[96:119]    temporaries, per-buffer fragment addresses of the 3-buffer variants
+  inputs are pinned by the C++ wrapper to v[120:191] and s[28:55] (see GmmTileRegs).
 """
 import sys
 
@@ -73,19 +83,20 @@ STAGE_BYTES = 4 * 128 * PITCH
 # ---- fixed register map: one wave per SIMD (128 x 128 per wave, 256 accumulators), the wave owns all 512
 # registers of a lane.
 STAGES_SHORT = 3         # LDS buffers of the 128- and 64-row tiles
-V_AF = [0, 16]           # A fragment sets (4 x 4 registers each)
-V_BF = [32, 48]
-V_TMP = 64               # 64..95
-V_VOA_HEAD, V_VOB_HEAD, V_VOA, V_VOB, V_VOA_TAIL, V_VOB_TAIL = 128, 136, 144, 152, 160, 168
-V_RA, V_RB = 176, 180    # fragment read addresses (4 + 4)
-V_EPI = 184              # +0: stage write addr, +1: stage read addr, +2: store voffset, +3: row - row_lo
-V_OOB = 188              # constant 0x80000000
-V_EPI2 = 190             # +0: store voffset whatever the chunk's validity, +1: mask of valid elements if partial
-V_BUFA, V_BUFB = 98, 110  # three-buffer variants: fragment addresses per (buffer, step), 12 + 12
-V_FIX = 196              # A first-chunk addr, A last-chunk addr, same for B (buffer 0)
-V_TOUCH = 192            # per-lane offsets of the L2 prefetch touches: +0 A, +1 B (K tile 0)
-V_TOUCH_DST = 96         # +0 / +1: where the touched dwords land (never read)
-V_CLOBBER = 122
+V_AF = [0, 16]           # A fragment sets (up to 4 fragments x 4 registers each)
+V_BF = [32, 64]          # B fragment sets (8 x 4 registers each)
+V_TMP = 96               # 96..105: temporaries of the main loop (the epilogue uses the fragment registers)
+V_TOUCH_DST = V_TMP + 10  # +0 / +1: where the touched dwords land (never read)
+V_BUFA, V_BUFB = V_TMP + 12, V_TMP + 18  # three-buffer variants: fragment addresses per (buffer, k half), 6 + 6
+V_CLOBBER = 120
+V_IN = 120               # first register of the inputs the wrapper pins
+V_VOA_HEAD, V_VOB_HEAD, V_VOA, V_VOB, V_VOA_TAIL, V_VOB_TAIL = (V_IN + 8 * i for i in range(6))
+V_RA, V_RB = V_IN + 48, V_IN + 52   # fragment read addresses (K-contiguous operand: one per k half; else one)
+V_EPI = V_IN + 56        # +0: stage write addr, +1: stage read addr, +2: store voffset, +3: row - row_lo
+V_OOB = V_IN + 60        # constant 0x80000000
+V_EPI2 = V_IN + 62       # +0: store voffset whatever the chunk's validity, +1: mask of valid elements if partial
+V_TOUCH = V_IN + 64      # per-lane offsets of the L2 prefetch touches: +0 A, +1 B (K tile 0)
+V_FIX = V_IN + 68        # A first-chunk addr, A last-chunk addr, same for B (buffer 0)
 S_MASK = 28            # s[28:31] keep-mask of the first chunk of the k range, s[32:35] of the last chunk
 
 S_RA, S_RB, S_RC = 36, 40, 44   # buffer resources
@@ -117,7 +128,8 @@ def sr(base, n=1):
 
 
 class Variant:
-    """tm = MFMA block rows per wave: the tile is 64 tm rows (256 / 128 / 64) by 256 columns."""
+    """tm = 32-row blocks per wave: the tile is 64 tm rows (256 / 128 / 64) by 256 columns; a wave computes
+    2 tm x 8 MFMA blocks of 16 x 16."""
 
     def __init__(self, a_tr, b_tr, out_f32, tm=4, f16=0, b_nt=0, act=0):
         """b_nt: B is copied with the non-temporal hint (a B panel that no other tile reads).
@@ -129,7 +141,7 @@ class Variant:
         assert not (self.act and (out_f32 or a_tr)) and not (self.partial and (not out_f32 or b_nt))
         self.dt = "f16" if f16 else "bf16"   # element type of A, B and of a 16-bit output
         assert tm in (1, 2, 4) and (tm == 4 or not a_tr)
-        self.tn = 4                      # 32-column MFMA blocks per wave (the wave grid is 2 x 2)
+        self.tn = 8                      # 16-column MFMA blocks per wave (the wave grid is 2 x 2)
         self.na = 2 * tm                 # copies of the A tile per wave and K tile
         self.nb = 8                      # ... of the B tile
         self.ncopy = self.na + self.nb
@@ -157,62 +169,64 @@ class Variant:
                                             "_bnt" if b_nt else "", "_swiglu" if act == 1 else ("_partial" if act == 2 else ""))
 
     def acc(self, i, j):
-        return (self.tn * i + j) * 16
+        """First accumulator register of the wave's 16 x 16 block (i, j), i < 2 tm, j < 8."""
+        return (self.tn * i + j) * 4
 
-    # -- fragment reads of k16 step `s` of buffer `buf` into register set `st`; returns list of instr
-    def frag_reads(self, buf, s, st):
-        """Order: A block 0, all B blocks, then the other A blocks -- the order in which the MFMAs of the
-        step (block row 0 first) need them, so that they can start while later reads are still in flight."""
-        blocks = {}
-        for op, tr, vbase, vaddr, vbuf, stage, nblk in (
-            ("A", self.a_tr, V_AF[st], V_RA, V_BUFA, self.a_stage, self.tm),
-            ("B", self.b_tr, V_BF[st], V_RB, V_BUFB, self.b_stage, self.tn),
-        ):
-            # two buffers: the buffer is an immediate offset; three: one address register per buffer and
-            # step (set up by the prologue), because the offsets no longer fit the 16-bit immediate
-            if self.stages == 2:
-                reg, boff = (vaddr + s if not tr else vaddr), buf * stage
-            else:
-                reg, boff = (vbuf + 4 * buf + s if not tr else vbuf + 4 * buf), 0
-            for x in range(nblk):
-                d = vbase + 4 * x
-                if not tr:
-                    # address register per step; sub-tiles are 32 rows = 4096 bytes apart
-                    blocks[(op, x)] = ["ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(reg), boff + x * 4096)]
-                else:
-                    o = boff + s * 8 * TR_BLOCK + x * 64
-                    blocks[(op, x)] = ["ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d, 2), vr(reg), o),
-                                       "ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d + 2, 2), vr(reg), o + 512)]
-        self.read_order = [("A", 0)] + [("B", x) for x in range(self.tn)] + [("A", x) for x in range(1, self.tm)]
-        self.read_len = {t: len(blocks[t]) for t in self.read_order}
+    # -- one fragment (16 rows or columns x 32 k) of k half `sp` of buffer `buf` into registers d .. d + 3;
+    # f = 16-row block of the wave's rows (A) / 16-column block of its columns (B)
+    def frag_read(self, is_a, buf, sp, f, d):
+        tr = self.a_tr if is_a else self.b_tr
+        stage = self.a_stage if is_a else self.b_stage
+        vaddr, vbuf = (V_RA, V_BUFA) if is_a else (V_RB, V_BUFB)
+        # two buffers: the buffer is an immediate offset; three: one address register per buffer (and k
+        # half), set up by the prologue, because the offsets no longer fit the 16-bit immediate
+        if not tr:
+            # address register per k half; 16-row blocks are 2048 bytes apart
+            reg, off = (vaddr + sp, buf * stage) if self.stages == 2 else (vbuf + 2 * buf + sp, 0)
+            return ["ds_read_b128 %s, %s offset:%d" % (vr(d, 4), vr(reg), off + f * 2048)]
+        reg, off = (vaddr, buf * stage) if self.stages == 2 else (vbuf + 2 * buf, 0)
+        o = off + sp * 16 * TR_BLOCK + f * 32
+        return ["ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d, 2), vr(reg), o),
+                "ds_read_b64_tr_b16 %s, %s offset:%d" % (vr(d + 2, 2), vr(reg), o + 512)]
+
+    def a_reads(self, buf, t, order=None):
+        """A fragments of step t (k half t / 2, row half t % 2) into A set t % 2: list of (tag, instructions)."""
+        sp, h, st = t // 2, t % 2, t % 2
+        return [(("A", st, x), self.frag_read(True, buf, sp, h * self.tm + x, V_AF[st] + 4 * x)) for x in range(self.tm)]
+
+    def b_reads(self, buf, sp, js):
+        """B fragments js of k half sp into B set sp."""
+        return [(("B", sp, j), self.frag_read(False, buf, sp, j, V_BF[sp] + 4 * j)) for j in js]
+
+    def first_reads(self, buf):
+        """What step 0 of a K tile on `buf` needs, in the order its MFMAs want it: issued by the prologue and by
+        step 3 of the K tile before."""
+        a, b = self.a_reads(buf, 0), self.b_reads(buf, 0, range(self.tn))
+        return a[:1] + b + a[1:]
+
+    def step_reads(self, t, buf, nb):
+        """Fragment reads issued during step t of a K tile on buffer `buf` (nb = buffer of the next K tile)."""
+        if t == 0:
+            return self.a_reads(buf, 1) + self.b_reads(buf, 1, range(0, 4))
+        if t == 1:
+            a = self.a_reads(buf, 2)
+            return a[:1] + self.b_reads(buf, 1, range(4, 8)) + a[1:]
+        if t == 2:
+            return self.a_reads(buf, 3)
+        return self.first_reads(nb)
+
+    # -- MFMAs of step t: list of (operand tags, instruction)
+    def mfmas(self, t):
+        sp, h, st = t // 2, t % 2, t % 2
         out = []
-        for t in self.read_order:
-            out += blocks[t]
-        return out
-
-    def read_need(self):
-        """For every MFMA of a step (in mfmas() order): how many of the step's fragment reads, in issue
-        order, must have completed before it; and the number of reads of a step."""
-        self.frag_reads(0, 0, 0)
-        end, n = {}, 0
-        for t in self.read_order:
-            n += self.read_len[t]
-            end[t] = n
-        return [max(end[("A", i)], end[("B", j)]) for i in range(self.tm) for j in range(self.tn)], n
-
-    def n_frag_reads(self):
-        return 4 * (2 if self.a_tr else 1) + 4 * (2 if self.b_tr else 1)
-
-    # -- MFMAs of one step on register set st
-    def mfmas(self, st):
-        out = []
-        for i in range(self.tm):
+        for x in range(self.tm):
+            i = h * self.tm + x
             for j in range(self.tn):
-                a = vr(V_AF[st] + 4 * i, 4)
-                b = vr(V_BF[st] + 4 * j, 4)
-                c = "a[%d:%d]" % (self.acc(i, j), self.acc(i, j) + 15)
+                a = vr(V_AF[st] + 4 * x, 4)
+                b = vr(V_BF[sp] + 4 * j, 4)
+                c = "a[%d:%d]" % (self.acc(i, j), self.acc(i, j) + 3)
                 # operands swapped: the result block is transposed, a lane owns 4 consecutive columns of a row
-                out.append("v_mfma_f32_32x32x16_%s %s, %s, %s, %s" % (self.dt, c, b, a, c))
+                out.append(((("A", st, x), ("B", sp, j)), "v_mfma_f32_16x16x32_%s %s, %s, %s, %s" % (self.dt, c, b, a, c)))
         return out
 
     # -- copy instruction with issue index n (0..15) of a K tile into buffer buf.
@@ -296,38 +310,53 @@ def fixup(e, v, which, buf):
         e("ds_write_b128 %s, %s" % (vr(ta), vr(t, 4)))
 
 
-def interleave(e, mfmas, side_groups, need=None, prev_total=0):
-    """Emit the MFMAs of a step with the side groups spread between them (after each MFMA, in order).  A
-    group that starts with a write of m0 has that write moved in front of the MFMA, which then is the
-    instruction the hardware wants between the write and the copy.
+class LdsOrder:
+    """LDS reads complete in the order they were issued.  Tracks the reads that may still be in flight, so that
+    an MFMA waits (s_waitcnt lgkmcnt) only until its own operands have arrived."""
 
-    need / prev_total: the operands of MFMA k are the first need[k] of the prev_total LDS reads issued
-    before this step (LDS reads complete in order); each MFMA waits only for those, counting the reads
-    this step has issued in the meantime (lgkmcnt has 4 bits: a larger allowance waits for 15)."""
+    def __init__(self, pending=()):
+        self.pending = list(pending)       # tags, oldest first
+
+    def issue(self, tag, n=1):
+        self.pending += [tag] * n
+
+    def wait_for(self, tags):
+        """The wait that proves every read with one of `tags` complete, or None if they already are."""
+        idx = max((i for i, t in enumerate(self.pending) if t in tags), default=-1)
+        if idx < 0:
+            return None
+        w = min(len(self.pending) - 1 - idx, 15)   # the counter has 4 bits
+        self.pending = self.pending[len(self.pending) - w:] if w else []
+        return w
+
+    def clear(self):
+        self.pending = []
+
+
+def interleave(e, lds, mfmas, side):
+    """Emit the MFMAs of a step with the side groups spread between them (after each MFMA, in order).  A
+    side group is (tag, instructions): tag names the fragment a group of LDS reads fetches (None: not a
+    read).  A group that starts with a write of m0 has that write moved in front of the MFMA, which then is
+    the instruction the hardware wants between the write and the copy."""
     n = len(mfmas)
     slots = [[] for _ in range(n)]
-    # spread groups evenly over the first n - 1 gaps
-    g = len(side_groups)
-    for k, grp in enumerate(side_groups):
-        slots[min(n - 1, (k * n) // max(g, 1))].extend(grp)
+    g = len(side)
+    for k, grp in enumerate(side):
+        slots[min(n - 1, (k * n) // max(g, 1))].append(grp)
     lines = []
-    bound = 1 << 30   # upper bound on the LDS reads in flight, as far as the emitted waits prove it
-    issued = 0        # reads issued in this step so far
     for k in range(n):
-        side = list(slots[k])
-        if side and side[0].startswith("s_add_u32 m0"):
-            lines.append(side.pop(0))
-        if need is not None:
-            allowed = prev_total - need[k] + issued
-            if bound > allowed:
-                w = min(allowed, 15)
-                lines.append("s_waitcnt lgkmcnt(%d)" % w)
-                bound = w
-        lines.append(mfmas[k])
-        lines.extend(side)
-        nr = sum(1 for x in side if x.startswith("ds_read"))
-        issued += nr
-        bound += nr
+        deps, ins = mfmas[k]
+        groups = [(tag, list(instrs)) for tag, instrs in slots[k]]
+        if groups and groups[0][1] and groups[0][1][0].startswith("s_add_u32 m0"):
+            lines.append(groups[0][1].pop(0))
+        w = lds.wait_for(deps)
+        if w is not None:
+            lines.append("s_waitcnt lgkmcnt(%d)" % w)
+        lines.append(ins)
+        for tag, instrs in groups:
+            lines.extend(instrs)
+            if tag is not None:
+                lds.issue(tag, sum(1 for x in instrs if x.startswith("ds_read")))
     for ins in m0_gaps(lines):
         e(ins)
 
@@ -380,8 +409,8 @@ def gen_main(v, e, L):
             stage = v.a_stage if is_a else v.b_stage
             src, dst = (V_RA, V_BUFA) if is_a else (V_RB, V_BUFB)
             for buf in range(S):
-                for st in range(1 if tr else 4):
-                    e("v_add_u32 %s, %d, %s" % (vr(dst + 4 * buf + st), buf * stage, vr(src + st)))
+                for sp in range(1 if tr else 2):
+                    e("v_add_u32 %s, %d, %s" % (vr(dst + 2 * buf + sp), buf * stage, vr(src + sp)))
     # tiles 1 .. S - 2 -> their buffers in full, tile S - 1 -> buffer S - 1: the first c3 copies
     slots = [(s_tail1, s_oob1, s_ka1, s_kb1), (s_tail2, s_oob2, s_ka2, s_kb2)]
     for tix in range(1, S):
@@ -406,7 +435,7 @@ def gen_main(v, e, L):
                     e(ins)
                 n_pro_touch += 1
     # zero the accumulators while the copies fly
-    for r in range(16 * v.tm * v.tn):
+    for r in range(64 * v.tm):
         e("v_accvgpr_write_b32 a%d, 0" % r)
     e("s_waitcnt vmcnt(%d)" % ((S - 2) * v.ncopy + c3 + n_pro_touch))
     e("s_barrier")
@@ -430,21 +459,24 @@ def gen_main(v, e, L):
         e("s_waitcnt lgkmcnt(0)")
         e("s_barrier")
         e.label("L_nofix0_%s" % L)
-    for ins in v.frag_reads(0, 0, 0):
-        e(ins)
+    for tag, instrs in v.first_reads(0):
+        for ins in instrs:
+            e(ins)
     e("s_mov_b32 %s, 0" % sr(s_kt))
     e("s_cmp_eq_u32 %s, 0" % sr(S_NK))
     e("s_cbranch_scc1 L_done_%s" % L)
 
     # ------------------------------------------------------------------ K loop, two tiles per trip
-    need, nreads = v.read_need()
+    def tagged(groups):
+        return [(None, g) for g in groups]
 
     def ktile(buf, fast):
-        # on entry: fragments of step 0 in set 0 (in flight); the first c3 copies of tile kt + S - 1 in flight.
+        # on entry: the fragments of step 0 are in flight (first_reads); the first c3 copies of tile kt + S - 1 too.
         # fast: tiles kt + S - 1 and kt + S are both before the last one, so their copies need neither the
         # tail offsets nor the out-of-range select, and tile kt + 1 cannot be the last one.
         which = "fast" if fast else "loop"
         e("; ---- k tile on buffer %d%s" % (buf, " (interior)" if fast else ""))
+        lds = LdsOrder(tag for tag, instrs in v.first_reads(buf) for _ in instrs)
         # K offsets (and masks) of tiles kt + S - 1 (copied during steps 0..2) and kt + S (step 3)
         e("s_add_u32 %s, %s, %d" % (sr(s_t1), sr(s_kt), S - 1))
         if not fast:
@@ -464,24 +496,25 @@ def gen_main(v, e, L):
             e("s_mul_i32 %s, %s, %s" % (sr(s_ktb), sr(s_t1), sr(S_BSTEP)))
         nb = (buf + 1) % S       # buffer of tile kt + 1
         cb = (buf + S - 1) % S   # buffer of tile kt + S - 1
-        # step 0: MFMA set 0, read step 1 -> set 1, next copies of tile kt + S - 1
-        side = [[x] for x in v.frag_reads(buf, 1, 1)]
-        side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)]
-        interleave(e, v.mfmas(0), side, need, nreads)
+        # step 0: the reads of step 1 (and half of the B fragments of k 32..63), next copies of tile kt + S - 1
+        side = v.step_reads(0, buf, nb)
+        side += tagged(v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0))
+        interleave(e, lds, v.mfmas(0), side)
         # step 1
-        side = [[x] for x in v.frag_reads(buf, 2, 0)]
-        side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)]
+        side = v.step_reads(1, buf, nb)
+        side += tagged(v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1))
         # the touches come after every copy of tile kt + S - 1 in issue order (c1 == c2 == 0), so the wait below
         # can leave them in flight: they have until the next K tile's wait to land
         assert c1 == 0 and c2 == 0
-        side += [touch_group(v, op, s_tmask, s_kta if op == "a" else s_ktb, V_TMP + 8 + k) for k, op in enumerate(v.touch)]
-        interleave(e, v.mfmas(1), side, need, nreads)
+        side += tagged(touch_group(v, op, s_tmask, s_kta if op == "a" else s_ktb, V_TMP + 8 + k) for k, op in enumerate(v.touch))
+        interleave(e, lds, v.mfmas(1), side)
         # step 2
-        side = [[x] for x in v.frag_reads(buf, 3, 1)]
-        side += [v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)]
-        interleave(e, v.mfmas(0), side, need, nreads)
+        side = v.step_reads(2, buf, nb)
+        side += tagged(v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy))
+        interleave(e, lds, v.mfmas(2), side)
         # tile kt+1 has landed for this wave; after the barrier for all, and `buf` is free
         e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % ((S - 2) * (v.ncopy + v.nt) + v.nt))
+        lds.clear()
         e("s_barrier")
         if not (v.a_tr and v.b_tr) and not fast:
             # the tile that has just landed is the last one and its last chunk is partial
@@ -494,10 +527,10 @@ def gen_main(v, e, L):
             e("s_waitcnt lgkmcnt(0)")
             e("s_barrier")
             e.label("L_nofix%d_%s" % (buf + 1, L))
-        # step 3: MFMA set 1, read step 0 of the next tile -> set 0, first copies of tile kt + S -> buf
-        side = [[x] for x in v.frag_reads(nb, 0, 0)]
-        side += [v.dma(n, buf, which, s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, c3)]
-        interleave(e, v.mfmas(1), side)
+        # step 3: the first fragments of the next tile, first copies of tile kt + S -> buf
+        side = v.step_reads(3, buf, nb)
+        side += tagged(v.dma(n, buf, which, s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, c3))
+        interleave(e, lds, v.mfmas(3), side)
         e("s_add_u32 %s, %s, 1" % (sr(s_kt), sr(s_kt)))
 
     def ktile_both(buf):
@@ -531,8 +564,8 @@ def gen_variant(v):
 
 def gen_epilogue(v, e, L):
     """Accumulators -> output.  The MFMA operands are swapped, so a lane owns 4 consecutive columns of a
-    row: acc block (i, j), register 4 q + r  ->  C[m = 32 i + lane % 32][n = 32 j + 8 q + 4 (lane / 32) + r].
-    The wave stages its block in LDS (rows padded to `pitch` bytes; `ipp` MFMA block rows per pass: all of
+    row: acc block (i, j), register r  ->  C[m = 16 i + lane % 16][n = 16 j + 4 (lane / 16) + r].
+    The wave stages its block in LDS (rows padded to `pitch` bytes; `ipp` groups of 32 rows per pass: all of
     them for a 16-bit output, one for fp32, whose rows are twice as long) and reads it back so that each lane
     holds 16 consecutive bytes of a row: every store instruction writes whole rows of the wave's 128 columns
     (256 contiguous bytes of 4 rows, or 512 contiguous bytes of 2 rows for fp32).
@@ -546,13 +579,13 @@ def gen_epilogue(v, e, L):
     e("s_nop 15")
     e("s_nop 15")
     e("s_barrier")
-    t = V_TMP
+    t = 0                                 # temporaries of the epilogue: the fragment registers
     f32 = v.out_f32
     esz = 4 if f32 else 2
     nel = 16 // esz                       # elements of a 16-byte chunk
     pitch = PITCH32 if f32 else (PITCH_ACT if v.act else PITCH)
-    ipp = 1 if f32 else v.tm              # MFMA block rows per pass
-    ncol = 64 if v.act else 32 * v.tn     # elements of a staged row
+    ipp = 1 if f32 else v.tm              # groups of 32 rows (two MFMA block rows) per pass
+    ncol = 64 if v.act else 16 * v.tn     # elements of a staged row
     rpi = 1024 // (ncol * esz)            # rows per read-back instruction (64 lanes x 16 bytes)
     depth = 4
     regs = [t + 4 * x for x in range(depth)]          # read-back data, 4 registers each
@@ -573,50 +606,49 @@ def gen_epilogue(v, e, L):
     nstore = 0
     for p0 in range(0, v.tm, ipp):
         k = 0
-        for il in range(min(ipp, v.tm - p0)):
-            i = p0 + il
+        for il2 in range(2 * min(ipp, v.tm - p0)):
+            i = 2 * p0 + il2                   # MFMA block row of the wave
+            rowoff = 16 * il2 * pitch          # its first row in the staging area
             if v.act:
-                # silu(g) * u = g * u / (1 + 2^(-g log2 e)); gate block j pairs with block j + 2 (64 columns on).
+                # silu(g) * u = g * u / (1 + 2^(-g log2 e)); gate block j pairs with block j + 4 (64 columns on).
                 # Four elements advance together, so no result of a transcendental is read by the next instruction.
-                for j in range(2):
-                    for q in range(4):
-                        b = t + 12 * (k % 2)
-                        k += 1
-                        g0, u0 = v.acc(i, j) + 4 * q, v.acc(i, j + 2) + 4 * q
-                        for r in range(4):
-                            e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), g0 + r))
-                        for r in range(4):
-                            e("v_accvgpr_read_b32 %s, a%d" % (vr(b + 4 + r), u0 + r))
-                        for r in range(4):
-                            e("v_mul_f32 %s, 0xbfb8aa3b, %s" % (vr(b + 8 + r), vr(b + r)))
-                        for r in range(4):
-                            e("v_exp_f32 %s, %s" % (vr(b + 8 + r), vr(b + 8 + r)))
-                        e("s_nop 0")
-                        for r in range(4):
-                            e("v_add_f32 %s, 1.0, %s" % (vr(b + 8 + r), vr(b + 8 + r)))
-                        for r in range(4):
-                            e("v_rcp_f32 %s, %s" % (vr(b + 8 + r), vr(b + 8 + r)))
-                        for r in range(4):
-                            e("v_mul_f32 %s, %s, %s" % (vr(b + r), vr(b + r), vr(b + 4 + r)))
-                        for r in range(4):
-                            e("v_mul_f32 %s, %s, %s" % (vr(b + r), vr(b + r), vr(b + 8 + r)))
-                        e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 8), vr(b), vr(b + 1)))
-                        e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 9), vr(b + 2), vr(b + 3)))
-                        e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 8, 2), (32 * il) * pitch + (32 * j + 8 * q) * 2))
+                for j in range(4):
+                    b = t + 12 * (k % 2)
+                    k += 1
+                    g0, u0 = v.acc(i, j), v.acc(i, j + 4)
+                    for r in range(4):
+                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), g0 + r))
+                    for r in range(4):
+                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b + 4 + r), u0 + r))
+                    for r in range(4):
+                        e("v_mul_f32 %s, 0xbfb8aa3b, %s" % (vr(b + 8 + r), vr(b + r)))
+                    for r in range(4):
+                        e("v_exp_f32 %s, %s" % (vr(b + 8 + r), vr(b + 8 + r)))
+                    e("s_nop 0")
+                    for r in range(4):
+                        e("v_add_f32 %s, 1.0, %s" % (vr(b + 8 + r), vr(b + 8 + r)))
+                    for r in range(4):
+                        e("v_rcp_f32 %s, %s" % (vr(b + 8 + r), vr(b + 8 + r)))
+                    for r in range(4):
+                        e("v_mul_f32 %s, %s, %s" % (vr(b + r), vr(b + r), vr(b + 4 + r)))
+                    for r in range(4):
+                        e("v_mul_f32 %s, %s, %s" % (vr(b + r), vr(b + r), vr(b + 8 + r)))
+                    e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 8), vr(b), vr(b + 1)))
+                    e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 9), vr(b + 2), vr(b + 3)))
+                    e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 8, 2), rowoff + 16 * j * 2))
                 continue
             for j in range(v.tn):
-                for q in range(4):
-                    b = t + 6 * (k % 4)
-                    k += 1
-                    a0 = v.acc(i, j) + 4 * q
-                    for r in range(4):
-                        e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), a0 + r))
-                    if f32:
-                        e("ds_write_b128 %s, %s offset:%d" % (vr(V_EPI), vr(b, 4), (32 * il) * pitch + (32 * j + 8 * q) * 4))
-                    else:
-                        e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 4), vr(b), vr(b + 1)))
-                        e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 5), vr(b + 2), vr(b + 3)))
-                        e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 4, 2), (32 * il) * pitch + (32 * j + 8 * q) * 2))
+                b = t + 6 * (k % 4)
+                k += 1
+                a0 = v.acc(i, j)
+                for r in range(4):
+                    e("v_accvgpr_read_b32 %s, a%d" % (vr(b + r), a0 + r))
+                if f32:
+                    e("ds_write_b128 %s, %s offset:%d" % (vr(V_EPI), vr(b, 4), rowoff + 16 * j * 4))
+                else:
+                    e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 4), vr(b), vr(b + 1)))
+                    e("v_cvt_pk_%s_f32 %s, %s, %s" % (v.dt, vr(b + 5), vr(b + 2), vr(b + 3)))
+                    e("ds_write_b64 %s, %s offset:%d" % (vr(V_EPI), vr(b + 4, 2), rowoff + 16 * j * 2))
         e("s_waitcnt lgkmcnt(0)")
         nrb = min(ipp, v.tm - p0) * 32 // rpi   # read-back instructions of this pass
         for r in range(min(depth, nrb)):
@@ -660,7 +692,7 @@ def gen_epilogue(v, e, L):
 def clobbers(v):
     c = ["memory", "vcc", "scc"]
     c += ["v%d" % i for i in range(0, V_CLOBBER)] + ["v%d" % V_OOB]
-    c += ["a%d" % i for i in range(16 * 4 * v.tn)]
+    c += ["a%d" % i for i in range(256)]
     c += ["s%d" % i for i in range(S_T, S_T + 34)]
     return ", ".join('"%s"' % x for x in c)
 
@@ -695,9 +727,11 @@ def main():
             out.append("  asm volatile(")
             out.append(e.text())
             out.append("      :")
-            out.append('      : "{v[128:135]}"(r.voa_head), "{v[136:143]}"(r.vob_head), "{v[144:151]}"(r.voa), "{v[152:159]}"(r.vob),')
-            out.append('        "{v[160:167]}"(r.voa_tail), "{v[168:175]}"(r.vob_tail), "{v[176:179]}"(r.ra_addr), "{v[180:183]}"(r.rb_addr),')
-            out.append('        "{v[184:187]}"(r.epi), "{v[190:191]}"(r.epi2), "{v[192:193]}"(r.touch), "{v[196:199]}"(r.fix), "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
+            pins = [(V_VOA_HEAD, 8, "voa_head"), (V_VOB_HEAD, 8, "vob_head"), (V_VOA, 8, "voa"), (V_VOB, 8, "vob"),
+                    (V_VOA_TAIL, 8, "voa_tail"), (V_VOB_TAIL, 8, "vob_tail"), (V_RA, 4, "ra_addr"), (V_RB, 4, "rb_addr"),
+                    (V_EPI, 4, "epi"), (V_EPI2, 2, "epi2"), (V_TOUCH, 2, "touch"), (V_FIX, 4, "fix")]
+            out.append("      : " + ", ".join('"{v[%d:%d]}"(r.%s)' % (b0, b0 + n - 1, name) for b0, n, name in pins) + ",")
+            out.append('        "{s[28:35]}"(r.masks), "{s[36:39]}"(r.rsrc_a), "{s[40:43]}"(r.rsrc_b), "{s[44:47]}"(r.rsrc_c), "{s[48:55]}"(r.scal)')
             out.append("      : %s);" % clobbers(v))
             out.append("}")
     sys.stdout.write("\n".join(out) + "\n")

@@ -172,21 +172,29 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   GmmTileRegs r;
   gmm_copy_offsets<A_TR, 2 * TM>(lane, wave, t.a, t.klen, t.khead, nk, r.voa_head, r.voa, r.voa_tail);
   gmm_copy_offsets<B_TR, 8>(lane, wave, t.b, t.klen, t.khead, nk, r.vob_head, r.vob, r.vob_tail);
+  // Fragment read addresses.  An MFMA fragment is 16 rows (or columns) x 32 k: lane l holds row l % 16,
+  // k 8 (l / 16) .. + 7.  K-contiguous operand: one ds_read_b128 of chunk 4 sp + l / 16 of the lane's row
+  // (sp = k half of the K tile; one address per half, 16-row blocks are immediate offsets).  Transposed
+  // layout: two ds_read_b64_tr_b16, each a 4 (k) x 16 (rows) block whose 16 lanes address 4 consecutive
+  // rows of k row ii / 4; k rows 8 q .. 8 q + 3 are the first rows of LDS blocks 4 q .. 4 q + 3 (k halves,
+  // 16-row blocks and the second four k rows are immediate offsets).
   const int q = lane >> 4, ii = lane & 15;
+  r.ra_addr = gmm_v4i{0, 0, 0, 0};
+  r.rb_addr = gmm_v4i{0, 0, 0, 0};
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const int chunk = 2 * s + (lane >> 5);
+  for (int sp = 0; sp < 2; ++sp) {
+    const int chunk = 4 * sp + q;
     if (!A_TR) {
-      const int row = wm * WROWS + (lane & 31);
-      r.ra_addr[s] = lds_base + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
-    } else {
-      r.ra_addr[s] = lds_base + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wm * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
+      const int row = wm * WROWS + ii;
+      r.ra_addr[sp] = lds_base + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
+    } else if (sp == 0) {
+      r.ra_addr[0] = lds_base + (4 * q + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wm * 128 + 4 * (ii & 3)) * 2;
     }
     if (!B_TR) {
-      const int row = wn * 128 + (lane & 31);
-      r.rb_addr[s] = lds_base + B_BASE + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
-    } else {
-      r.rb_addr[s] = lds_base + B_BASE + (4 * (q >> 1) + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wn * 128 + 16 * (q & 1) + 4 * (ii & 3)) * 2;
+      const int row = wn * 128 + ii;
+      r.rb_addr[sp] = lds_base + B_BASE + row * 128 + ((chunk ^ gmm_swz(row)) << 4);
+    } else if (sp == 0) {
+      r.rb_addr[0] = lds_base + B_BASE + (4 * q + (ii >> 2)) * GMM_TILE_TR_BLOCK + (wn * 128 + 4 * (ii & 3)) * 2;
     }
   }
   // Epilogue: the wave stages its block in LDS and reads it back row by row, 16 bytes per lane (see
@@ -200,7 +208,7 @@ __device__ __forceinline__ void gmm_tile_compute(const GmmTileDesc& t, unsigned 
   {
     const int row_t = wm * WROWS + lane / LPR, col_t = wn * WCOLS + (lane % LPR) * NEL;
     const unsigned stage = lds_base + wave * (STAGE_ROWS * EPITCH);
-    r.epi[0] = stage + (lane & 31) * EPITCH + 4 * ESZ * (lane >> 5);        // write: row lane % 32, columns 4 (lane / 32) ..
+    r.epi[0] = stage + (lane & 15) * EPITCH + 4 * ESZ * (lane >> 4);        // write: row lane % 16, columns 4 (lane / 16) ..
     r.epi[1] = stage + (lane / LPR) * EPITCH + (lane % LPR) * 16;           // read: row lane / LPR, chunk lane % LPR
     // the lane's columns: all valid -> one 16-byte store; some valid (a group boundary inside the chunk)
     // -> element stores under the mask; none -> nothing
