@@ -26,7 +26,7 @@ operands drawn like the benchmark's it sustains 1960-2050 TFLOP/s where
   * an operand that is contiguous along K lives in LDS as [row][64 k] with its
     16-byte chunks XOR-swizzled (conflict-free ds_read_b128 fragments); one that
     is contiguous along M / N lives as [k][256] in blocks of two k rows with a
-    64-byte pad, read with ds_read_b64_tr_b16 (the LDS transposes 4 x 16 blocks);
+    32-byte pad, read with ds_read_b64_tr_b16 (the LDS transposes 4 x 16 blocks);
   * a K tile is four steps: (k 0..31, upper half of the wave's rows), (k 0..31,
     lower half), (k 32..63, upper), (k 32..63, lower).  A step issues 8 tm
     v_mfma_f32_16x16x32 (tm = 4 for the 256-row tile) and, between them, the
@@ -75,7 +75,8 @@ TOUCH_OPS = "b"
 PITCH = 272           # bytes per staged row of 128 bf16 (256 + 16: shifts banks per row)
 PITCH32 = 528         # ... of 128 fp32 (512 + 16)
 PITCH_ACT = 144       # ... of the 64 gated values a wave's 128 columns give (128 + 16)
-TR_BLOCK = 1088       # two k rows of 512 bytes + 64 bytes pad
+TR_BLOCK = 1056       # two k rows of 512 bytes + 32 bytes pad: the four blocks that 16 lanes of a transposing read
+                      # address lie 8 banks apart (32 consecutive banks), the next 16 lanes' blocks on the other 32
 KC_STAGE = 256 * 64 * 2
 TR_STAGE = 32 * TR_BLOCK
 STAGE_BYTES = 4 * 128 * PITCH
@@ -243,8 +244,7 @@ class Variant:
         # per wave: 8 instructions of 1 KiB each; wave w covers [w * 8 KiB, (w + 1) * 8 KiB) of the
         # stage (row-chunk layout) or blocks w * 8 .. w * 8 + 7 (transposed layout): the wave part of
         # the LDS address is in s[S_T + 20] (A) / s[S_T + 21] (B), set up by the prologue.
-        blk = TR_BLOCK if tr else 1024
-        lds_off = lbase + buf * stage + i * blk
+        lds_off = lbase + buf * stage + i * (TR_BLOCK if tr else 1024)
         s_wave = S_T + 20 + (0 if is_a else 1)
         # m0 is written first: a write of m0 needs one other instruction before the copy that uses it
         # (the selects below, an MFMA that interleave() puts in between, or a s_nop)
@@ -470,6 +470,13 @@ def gen_main(v, e, L):
     def tagged(groups):
         return [(None, g) for g in groups]
 
+    def mix(reads, others):
+        """Both lists spread over the whole step, each keeping its order: the four waves of a workgroup issue
+        their copies at the same time, and bunched up they ask more of the address unit than it takes."""
+        keyed = [((i + 0.5) / len(reads), 0, i, g) for i, g in enumerate(reads)]
+        keyed += [((j + 0.5) / len(others), 1, j, g) for j, g in enumerate(others)]
+        return [g for _, _, _, g in sorted(keyed, key=lambda x: x[:3])]
+
     def ktile(buf, fast):
         # on entry: the fragments of step 0 are in flight (first_reads); the first c3 copies of tile kt + S - 1 too.
         # fast: tiles kt + S - 1 and kt + S are both before the last one, so their copies need neither the
@@ -497,20 +504,19 @@ def gen_main(v, e, L):
         nb = (buf + 1) % S       # buffer of tile kt + 1
         cb = (buf + S - 1) % S   # buffer of tile kt + S - 1
         # step 0: the reads of step 1 (and half of the B fragments of k 32..63), next copies of tile kt + S - 1
-        side = v.step_reads(0, buf, nb)
-        side += tagged(v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0))
+        side = mix(v.step_reads(0, buf, nb),
+                   tagged(v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3, c3 + c0)))
         interleave(e, lds, v.mfmas(0), side)
         # step 1
-        side = v.step_reads(1, buf, nb)
-        side += tagged(v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1))
-        # the touches come after every copy of tile kt + S - 1 in issue order (c1 == c2 == 0), so the wait below
-        # can leave them in flight: they have until the next K tile's wait to land
-        assert c1 == 0 and c2 == 0
-        side += tagged(touch_group(v, op, s_tmask, s_kta if op == "a" else s_ktb, V_TMP + 8 + k) for k, op in enumerate(v.touch))
+        side = mix(v.step_reads(1, buf, nb),
+                   tagged(v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0, c3 + c0 + c1)))
         interleave(e, lds, v.mfmas(1), side)
         # step 2
-        side = v.step_reads(2, buf, nb)
-        side += tagged(v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy))
+        side = mix(v.step_reads(2, buf, nb),
+                   tagged(v.dma(n, cb, which, s_tail1, s_oob1, s_ka1, s_kb1, V_TMP + (n % 8)) for n in range(c3 + c0 + c1, v.ncopy)))
+        # the touches come after every copy of tile kt + S - 1 in issue order, so the wait below can leave them
+        # in flight: they have until the next K tile's wait to land
+        side += tagged(touch_group(v, op, s_tmask, s_kta if op == "a" else s_ktb, V_TMP + 8 + k) for k, op in enumerate(v.touch))
         interleave(e, lds, v.mfmas(2), side)
         # tile kt+1 has landed for this wave; after the barrier for all, and `buf` is free
         e("s_waitcnt vmcnt(%d) lgkmcnt(0)" % ((S - 2) * (v.ncopy + v.nt) + v.nt))
@@ -528,8 +534,8 @@ def gen_main(v, e, L):
             e("s_barrier")
             e.label("L_nofix%d_%s" % (buf + 1, L))
         # step 3: the first fragments of the next tile, first copies of tile kt + S -> buf
-        side = v.step_reads(3, buf, nb)
-        side += tagged(v.dma(n, buf, which, s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, c3))
+        side = mix(v.step_reads(3, buf, nb),
+                   tagged(v.dma(n, buf, which, s_tail2, s_oob2, s_ka2, s_kb2, V_TMP + (n % 8)) for n in range(0, c3)))
         interleave(e, lds, v.mfmas(3), side)
         e("s_add_u32 %s, %s, 1" % (sr(s_kt), sr(s_kt)))
 
