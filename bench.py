@@ -223,42 +223,58 @@ def cpu_baseline(w, torch, budget_s=15.0):
             "sample": sample, "seconds": round(t, 3)}
 
 
-def mfma_only(args, torch, dev):
-    """Rate of the matrix pipe alone (register-only loop of the MFMA the kernels use), with operand values
-    drawn like the workload's (N(0,1) for A fragments, 0.02 N(0,1) for B fragments) and with zeros."""
+def load_diag():
+    """The bench-only diagnostics library (register-only MFMA loop), built beside the product library."""
     import ctypes
-    from grouped_mm_bf16_amd import _lib
-    lib = _lib.load()
+    from grouped_mm_bf16_amd import build
+    if not os.path.exists(build.DIAG_LIB_PATH):
+        raise SystemExit(f"{build.DIAG_LIB_PATH} is missing: build it with `python -m grouped_mm_bf16_amd.build`")
+    lib = ctypes.CDLL(build.DIAG_LIB_PATH)
+    i32, i64, vp = ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p
+    lib.gmm_diag_mfma_rate.restype = ctypes.c_int
+    lib.gmm_diag_mfma_rate.argtypes = [vp, i64, vp, i64, i32, i32, i32, vp, vp]
+    return lib
+
+
+def mfma_only(args, torch, dev):
+    """Rate of the matrix pipe alone (register-only loops of v_mfma_f32_16x16x32_bf16, which the assembly tile
+    uses, and of v_mfma_f32_32x32x16_bf16), with operand values drawn like the workload's (N(0,1) for A
+    fragments, 0.02 N(0,1) for B fragments) and with zeros."""
+    import ctypes
+    lib = load_diag()
     gen = torch.Generator().manual_seed(3)
     iters = 4000
     out = torch.empty(512 * 256 * 2, dtype=torch.float32, device=dev)
     res = {}
     for label, scale in (("random", 1.0), ("zeros", 0.0)):
-        # fragments alternate: 4 for A (unit scale), 4 for B (0.02), per thread
-        vals = torch.randn(4096, 8, generator=gen) * scale
-        vals[(torch.arange(4096) % 8) >= 4] *= 0.02
+        # 16 fragments per thread: the first 8 feed A operands (unit scale), the last 8 B operands (0.02)
+        vals = torch.randn(4096 * 16, 8, generator=gen) * scale
+        vals[(torch.arange(4096 * 16) % 16) >= 8] *= 0.02
         frags = vals.to(torch.bfloat16).to(dev)
-        for waves in (1, 2):
-            blocks = ctypes.c_int32(0)
+        for shape, shape_name in ((0, "16x16x32"), (1, "32x32x16")):
+            for waves in (1, 2):
+                blocks = ctypes.c_int32(0)
 
-            def launch():
-                _lib.check(lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), out.numel() * 4,
-                                                  waves, iters, ctypes.addressof(blocks),
-                                                  torch.cuda.current_stream().cuda_stream), "gmm_diag_mfma_rate")
-            for _ in range(args.warmup):
-                launch()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(args.steps):
-                launch()
-            e1.record()
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1) / args.steps
-            flops = blocks.value * 4 * iters * 16 * 32768.0
-            res[f"{label}_{waves}_waves_per_simd"] = round(flops / ms / 1e9, 1)
-    print(json.dumps({"metric": "v_mfma_f32_32x32x16_bf16 alone, register operands (context for the MFMA roofline)",
-                      "value": res["random_1_waves_per_simd"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+                def launch():
+                    rc = lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), out.numel() * 4,
+                                                waves, iters, shape, ctypes.addressof(blocks),
+                                                torch.cuda.current_stream().cuda_stream)
+                    if rc != 0:
+                        raise SystemExit(f"gmm_diag_mfma_rate failed with status {rc}")
+                for _ in range(args.warmup):
+                    launch()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(args.steps):
+                    launch()
+                e1.record()
+                torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1) / args.steps
+                flops = blocks.value * 4 * iters * 524288.0
+                res[f"{shape_name}_{label}_{waves}_waves_per_simd"] = round(flops / ms / 1e9, 1)
+    print(json.dumps({"metric": "v_mfma_f32_16x16x32_bf16 alone, register operands (context for the MFMA roofline)",
+                      "value": res["16x16x32_random_1_waves_per_simd"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
                       "warmup": args.warmup, "peak": PEAK_BF16_TFLOPS, "detail": res}))
 
 

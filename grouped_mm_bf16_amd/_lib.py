@@ -48,7 +48,6 @@ SIGNATURES = {
     "gmm_set_tile_heights": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     "gmm_set_tail_split": (ctypes.c_int, [ctypes.c_int]),
     "gmm_set_group_major": (ctypes.c_int, [ctypes.c_int]),
-    "gmm_diag_mfma_rate": (ctypes.c_int, [_vp, _i64, _vp, _i64, _i32, _i32, _vp, _vp]),
 }
 
 _lock = threading.Lock()

@@ -3,8 +3,9 @@
     python -m grouped_mm_bf16_amd.build [--force]
 
 Each .hip source under csrc/ is compiled to an object (in parallel) and the
-objects are linked into grouped_mm_bf16_amd/libgrouped_mm_hip.so.  hipcc
-cross-compiles, so no GPU is needed to build.
+objects are linked into grouped_mm_bf16_amd/libgrouped_mm_hip.so; csrc/diag/
+becomes libgmm_diag.so, which only bench.py loads.  hipcc cross-compiles, so no
+GPU is needed to build.
 """
 from __future__ import annotations
 
@@ -18,6 +19,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "csrc", "build")
 LIB_PATH = os.path.join(HERE, "libgrouped_mm_hip.so")
+# bench-only diagnostics (the register-only MFMA rate loop): a library of its own, loaded by bench.py alone
+DIAG_SRC = os.path.join(CSRC, "diag", "gmm_diag.hip")
+DIAG_LIB_PATH = os.path.join(HERE, "libgmm_diag.so")
 
 ARCH = "gfx950"
 FLAGS = [
@@ -86,8 +90,13 @@ def build(force: bool = False, verbose: bool = False) -> str:
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+    if force or _stale(DIAG_LIB_PATH, [DIAG_SRC]):
+        cmd = [_hipcc(), *FLAGS, "-shared", "-o", DIAG_LIB_PATH, DIAG_SRC]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {DIAG_SRC}:\n{res.stdout}\n{res.stderr}")
     if verbose:
-        print(f"built {LIB_PATH}")
+        print(f"built {LIB_PATH} and {DIAG_LIB_PATH}")
     return LIB_PATH
 
 

@@ -202,7 +202,10 @@ int gmm_moe_combine(const void* y, const int32_t* token_rows, const float* slot_
  * them, tests/test_grouped_mm.py:388-394).  gmm_set_path forces a kernel family
  * for later calls of this process and returns the previous setting;
  * gmm_last_path reports the family the calling thread's last launch used
- * (GMM_PATH_GENERIC or GMM_PATH_MFMA, 0 before any launch). */
+ * (GMM_PATH_GENERIC or GMM_PATH_MFMA, 0 before any launch).
+ * All gmm_set_* hooks below are process-wide and are not synchronised with launches
+ * of other threads (a launch that runs while another thread holds a forced setting
+ * takes that setting): they are for tests and tuning runs, not for serving code. */
 int gmm_set_path(int path);
 int gmm_last_path(void);
 /* Tile configuration of the MFMA family: -1 = choose from the shapes, 0 = register-staged kernel,
@@ -252,15 +255,6 @@ int64_t gmm_host_tile_list3(const int32_t* offs_host, int32_t G, int32_t jagged,
                             int32_t tall, int32_t shrt, int32_t tile_n, int32_t align,
                             int32_t xcd_remap, int32_t num_workgroups, int32_t max_parts,
                             int32_t group_major, int32_t* records, int64_t capacity);
-
-/* Diagnostic, no counterpart in the reference: launches a register-only loop of independent
- * v_mfma_f32_32x32x16_bf16 on every SIMD (waves_per_simd 1 or 2; 16 MFMAs of 32768 FLOP per wave and
- * iteration), with operand fragments taken from `frags` (device memory, frag_bytes >= 16, bf16 values of
- * the caller's choice: the sustained clock depends on them).  `out` receives one float per thread
- * (blocks * 256 floats); *blocks gets the number of 256-thread blocks launched, so that
- * FLOP per launch = *blocks * 4 * iters * 16 * 32768.  Returns a gmm_status. */
-int gmm_diag_mfma_rate(const void* frags, int64_t frag_bytes, void* out, int64_t out_bytes,
-                       int32_t waves_per_simd, int32_t iters, int32_t* blocks, void* stream);
 
 #ifdef __cplusplus
 }

@@ -331,20 +331,26 @@ def test_row_major_and_column_major_b_agree_bit_for_bit():
 
 
 def test_mfma_rate_diagnostic_runs():
-    """The register-only MFMA loop behind `bench.py --workload mfma_only`: argument checks and one launch."""
+    """The register-only MFMA loops behind `bench.py --workload mfma_only` (a bench-only library of their own):
+    argument checks and one launch per MFMA shape."""
     import ctypes
-    lib = K_._lib.load()
+    import bench
+    lib = bench.load_diag()
     frags = torch.randn(64, 8).to(torch.bfloat16).to(DEV)
     out = torch.full((512 * 256 * 2,), float("nan"), device=DEV)
     blocks = ctypes.c_int32(0)
     stream = torch.cuda.current_stream().cuda_stream
-    assert lib.gmm_diag_mfma_rate(None, 16, out.data_ptr(), out.numel() * 4, 1, 10, ctypes.addressof(blocks), stream) != 0
-    assert lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), 16, 1, 10, ctypes.addressof(blocks), stream) != 0
-    assert lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), out.numel() * 4, 2, 10,
-                                  ctypes.addressof(blocks), stream) == 0
-    torch.cuda.synchronize()
-    n = blocks.value * 256
-    assert blocks.value > 0 and torch.isfinite(out[:n]).all() and torch.isnan(out[n:]).all()
+    assert lib.gmm_diag_mfma_rate(None, 16, out.data_ptr(), out.numel() * 4, 1, 10, 0, ctypes.addressof(blocks), stream) != 0
+    assert lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), 16, 1, 10, 0, ctypes.addressof(blocks), stream) != 0
+    assert lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), out.numel() * 4, 1, 10, 2,
+                                  ctypes.addressof(blocks), stream) != 0
+    for shape in (0, 1):
+        out.fill_(float("nan"))
+        assert lib.gmm_diag_mfma_rate(frags.data_ptr(), frags.numel() * 2, out.data_ptr(), out.numel() * 4, 2, 10, shape,
+                                      ctypes.addressof(blocks), stream) == 0
+        torch.cuda.synchronize()
+        n = blocks.value * 256
+        assert blocks.value > 0 and torch.isfinite(out[:n]).all() and torch.isnan(out[n:]).all()
 
 
 @pytest.mark.parametrize("a_col", [False, True])
