@@ -332,3 +332,35 @@ def test_fine_grained_fixture_group_major_with_split(golden_dir):
     rec = tile_list3(sizes, ROWS, 32768, 768, 2048, 128, 64, 512, group_major=1)
     assert (rec[:, 11] == 1).all()          # 32 K tiles: too short a contraction to cut
     assert (coverage2(rec[:, :10], 128, 32768, 768, False) == 1).all()
+
+
+def fabric_floor_bytes(rec, K, num_wg=256, esz=2):
+    """Bytes the launch order must pull through the fabric if an XCD's L2 keeps an operand panel exactly as long
+    as the round that uses it: tiles are dealt round by round, workgroup w runs on XCD w % 8, and the tiles of
+    one XCD in one round share every A row panel (group, first row) and B column panel (group, first column)
+    they have in common.  Records in launch order, as gmm_host_tile_list2/3 return them."""
+    total = 0
+    for r0 in range(0, len(rec), num_wg):
+        span = rec[r0:r0 + num_wg]
+        for x in range(8):
+            mine = span[x::8]
+            a_panels = {(int(t[0]), int(t[1])): min(int(t[1]) + int(t[9]), int(t[4])) - max(int(t[1]), int(t[3])) for t in mine}
+            b_panels = {(int(t[0]), int(t[2])): min(int(t[2]) + 256, int(t[6])) - max(int(t[2]), int(t[5])) for t in mine}
+            total += (sum(a_panels.values()) + sum(b_panels.values())) * K * esz
+    return total
+
+
+def test_fabric_traffic_floor_of_the_mixtral_launch_order():
+    """What the 8 x 4 blocks per XCD must fetch past the L2s on the benchmark's headline workload: 3.47 GB of
+    operand panels for 1.07 GB of operands (every XCD reads all eight A panels of its band; a B panel is read by
+    one XCD per band of its group; a 2 MB panel outlives no round in a 4 MB L2).  The FETCH_SIZE counter reads
+    3.86 GB per launch on the device: 1.11 times this floor.  Without the XCD renumbering (a round's tiles dealt to the XCDs one by one)
+    every XCD touches every panel of the round: 2.6 times as much."""
+    def order(remap):
+        # device order: tile ids 0 .. n - 1 in launch order after the renumbering, workgroup w takes id w of a round
+        return tile_list3(MIXTRAL, ROWS, 16384, 14336, 4096, 256, 64, 0, remap=remap)
+    blocked, plain = fabric_floor_bytes(order(1), 4096), fabric_floor_bytes(order(0), 4096)
+    operands = (16384 * 4096 + 8 * 4096 * 14336) * 2
+    assert 3.4e9 < blocked < 3.55e9, blocked
+    assert plain > 2.4 * blocked
+    assert blocked > 2.5 * operands
