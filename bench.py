@@ -271,7 +271,7 @@ def mfma_only(args, torch, dev):
                 e1.record()
                 torch.cuda.synchronize()
                 ms = e0.elapsed_time(e1) / args.steps
-                flops = blocks.value * 4 * iters * 524288.0
+                flops = blocks.value * 4 * iters * (1048576.0 if shape == 0 else 524288.0)
                 res[f"{shape_name}_{label}_{waves}_waves_per_simd"] = round(flops / ms / 1e9, 1)
     print(json.dumps({"metric": "v_mfma_f32_16x16x32_bf16 alone, register operands (context for the MFMA roofline)",
                       "value": res["16x16x32_random_1_waves_per_simd"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,

@@ -39,7 +39,7 @@ __global__ void __launch_bounds__(256) diag_mfma_32x32x16(const diag_bf16x8* __r
   out[blockIdx.x * 256 + threadIdx.x] = r;
 }
 
-// one iteration = the same FLOPs as one iteration above: 64 MFMAs of 16384 FLOP = 16 of 32768
+// one iteration = 64 MFMAs of 16384 FLOP: twice the FLOPs of an iteration above (a k step of 32 instead of 16)
 __global__ void __launch_bounds__(256) diag_mfma_16x16x32(const diag_bf16x8* __restrict__ frags, int nfrags,
                                                           float* __restrict__ out, int iters) {
   diag_bf16x8 a[8], b[8];
@@ -68,7 +68,7 @@ __global__ void __launch_bounds__(256) diag_mfma_16x16x32(const diag_bf16x8* __r
 // frags: device memory, frag_bytes >= 16, bf16 values of the caller's choice, 16 fragments of 8 values per
 // thread (wrapping around): the first 8 feed the A operands, the last 8 the B operands.  `out` receives one
 // float per thread (blocks * 256 floats); *blocks gets the number of 256-thread blocks launched (one or two
-// waves on every SIMD), so that FLOP per launch = *blocks * 4 * iters * 524288.  Returns 0, 1 (bad argument)
+// waves on every SIMD), so that FLOP per launch = *blocks * 4 * iters * 1048576 for shape 0 and * 524288 for shape 1.  Returns 0, 1 (bad argument)
 // or 2 (launch failed).
 extern "C" int gmm_diag_mfma_rate(const void* frags, int64_t frag_bytes, void* out, int64_t out_bytes, int32_t waves_per_simd,
                                   int32_t iters, int32_t shape, int32_t* blocks_out, void* stream) {
