@@ -1,0 +1,138 @@
+"""Static check of the generated tile assembly (grouped_mm_bf16_amd/csrc/gen_tile_asm.py), no GPU needed.
+
+LDS reads complete in the order they were issued, and the generator puts in front of every MFMA the
+`s_waitcnt lgkmcnt(n)` that is meant to prove exactly its own operands.  This test replays the K loop of every
+variant instruction by instruction with that rule -- a read is known complete only once a wait has left fewer
+reads outstanding than were issued after it -- and fails if an MFMA could issue while one of its operand
+registers is still the destination of a read in flight, or if a read overwrites a fragment register that a
+later MFMA of the same step still wants with its old value."""
+import importlib.util
+import os
+import re
+
+import pytest
+
+ROOT = os.path.abspath(os.path.join(os.path.dirname(__file__), ".."))
+spec = importlib.util.spec_from_file_location("gen_tile_asm", os.path.join(ROOT, "grouped_mm_bf16_amd", "csrc", "gen_tile_asm.py"))
+gen = importlib.util.module_from_spec(spec)
+spec.loader.exec_module(gen)
+
+
+def regs(token):
+    """'v[4:7]' -> {4..7}, 'v12' -> {12}; anything else -> empty."""
+    m = re.fullmatch(r"v\[(\d+):(\d+)\]", token)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.fullmatch(r"v(\d+)", token)
+    return {int(m.group(1))} if m else set()
+
+
+def loop_bodies(variant):
+    """The K tile bodies of a variant as lists of instructions: {(buffer, interior?): [...]} and the prologue's tail."""
+    e = gen.Emit()
+    gen.gen_main(variant, e, "T")
+    bodies, cur, pro = {}, None, []
+    for line in e.lines:
+        m = re.match(r"; ---- k tile on buffer (\d+)( \(interior\))?", line)
+        if m:
+            cur = (int(m.group(1)), bool(m.group(2)))
+            bodies[cur] = []
+            continue
+        if cur is None:
+            pro.append(line)
+        elif line.startswith("s_branch L_join") or line.endswith(":") and line.startswith(("L_join", "L_slow", "L_done")):
+            cur = None if not line.startswith("L_slow") else cur
+            if line.startswith("L_slow"):
+                cur = None
+        elif line.startswith(("s_cmp", "s_cbranch")) and cur is not None and "L_nofix" not in line and bodies[cur] and \
+                bodies[cur][-1].startswith("s_add_u32 s56"):
+            cur = None          # the loop control after a body
+        else:
+            bodies[cur].append(line)
+    return pro, bodies
+
+
+class Lds:
+    def __init__(self):
+        self.queue = []           # destination register sets of the LDS operations in flight, oldest first
+
+    def busy(self):
+        return set().union(*self.queue) if self.queue else set()
+
+    def step(self, ins):
+        op, _, rest = ins.partition(" ")
+        args = [a.strip() for a in rest.split(",")]
+        if op.startswith("ds_read"):
+            self.queue.append(regs(args[0]))
+        elif op.startswith("ds_write"):
+            self.queue.append(set())
+        elif op == "s_waitcnt":
+            m = re.search(r"lgkmcnt\((\d+)\)", rest)
+            if m:
+                keep = int(m.group(1))
+                self.queue = self.queue[len(self.queue) - keep:] if keep else []
+        elif op == "s_barrier":
+            pass
+        elif op.startswith("v_mfma"):
+            srcs = regs(args[1]) | regs(args[2])
+            pending = self.busy() & srcs
+            assert not pending, f"{ins}: operand registers {sorted(pending)} may still be in flight"
+
+
+VARIANTS = [(a, b, tm) for a in (0, 1) for b in (0, 1) for tm in (4, 2, 1) if tm == 4 or not a]
+
+
+@pytest.mark.parametrize("a_tr,b_tr,tm", VARIANTS)
+def test_every_mfma_waits_for_its_own_operands(a_tr, b_tr, tm):
+    v = gen.Variant(a_tr, b_tr, 0, tm)
+    pro, bodies = loop_bodies(v)
+    stages = v.stages
+    assert sorted(bodies) == sorted((b, f) for b in range(stages) for f in (False, True))
+    for interior in (True, False):
+        lds = Lds()
+        # the prologue ends with the reads of step 0 of K tile 0; nothing before them matters here
+        first = [i for i, l in enumerate(pro) if l.startswith("ds_read")]
+        for ins in pro[first[0]:]:
+            lds.step(ins)
+        n_mfma = 0
+        for trip in range(2):                      # twice round the buffers: the second trip starts from the first's state
+            for buf in range(stages):
+                for ins in bodies[(buf, interior)]:
+                    lds.step(ins)
+                    n_mfma += ins.startswith("v_mfma")
+        assert n_mfma == 2 * stages * 32 * tm      # 8 tm MFMAs per step, four steps per K tile
+
+
+@pytest.mark.parametrize("a_tr,b_tr,tm", VARIANTS)
+def test_fragment_sets_alternate_so_that_no_read_lands_on_live_operands(a_tr, b_tr, tm):
+    """A read issued in a step must not target a register that an MFMA later in the same step still reads (the
+    hardware would be free to deliver it early)."""
+    v = gen.Variant(a_tr, b_tr, 0, tm)
+    _, bodies = loop_bodies(v)
+    for key, body in bodies.items():
+        # steps are delimited by the 8 tm MFMAs they hold
+        idx = [i for i, l in enumerate(body) if l.startswith("v_mfma")]
+        per = 8 * tm
+        assert len(idx) == 4 * per
+        for s in range(4):
+            lo = idx[s * per]
+            hi = idx[(s + 1) * per - 1]
+            for i in range(lo, hi):
+                if body[i].startswith("ds_read"):
+                    dst = regs(body[i].split(" ", 1)[1].split(",")[0].strip())
+                    for j in range(i + 1, hi + 1):
+                        if body[j].startswith("v_mfma"):
+                            a = [x.strip() for x in body[j].split(" ", 1)[1].split(",")]
+                            assert not dst & (regs(a[1]) | regs(a[2])), (key, body[i], body[j])
+
+
+def test_the_checker_catches_a_missing_wait():
+    """Sanity of the test itself: drop the waits and the replay must object."""
+    v = gen.Variant(0, 1, 0, 4)
+    pro, bodies = loop_bodies(v)
+    lds = Lds()
+    first = [i for i, l in enumerate(pro) if l.startswith("ds_read")]
+    with pytest.raises(AssertionError, match="may still be in flight"):
+        for ins in pro[first[0]:] + bodies[(0, True)]:
+            if not ins.startswith("s_waitcnt"):
+                lds.step(ins)
