@@ -300,36 +300,48 @@ __device__ __forceinline__ void gmm_split_finish(const GmmParams& p, char* c_gro
 #pragma unroll
   for (int e = 0; e < 4; ++e) valid |= (col + e >= n_lo && col + e < n_hi) ? (1 << e) : 0;
   if (valid == 0) return;
-  for (int r = r_begin + (tid >> 6); r < r_end; r += 4) {
-    const unsigned at_slot = unsigned(r * 256 + 4 * chunk) * 4;
-    float4 part[GMM_SPLIT_MAX];
+  // Four rows per thread at a time: their 4 * nparts loads are in flight together (each is a trip to the
+  // Infinity Cache or to memory; one row at a time, the loop is 64 such trips long).
+  constexpr int ROWS_AT_ONCE = 4;
+  for (int r0 = r_begin + (tid >> 6); r0 < r_end; r0 += 4 * ROWS_AT_ONCE) {
+    float4 part[ROWS_AT_ONCE][GMM_SPLIT_MAX];
 #pragma unroll
-    for (int j = 0; j < GMM_SPLIT_MAX; ++j)
-      if (j < nparts) part[j] = gmm_load_device_scope(slots, unsigned(j * tail) * unsigned(GMM_WS_SLOT) + at_slot);
-    float4 acc = part[0];
+    for (int u = 0; u < ROWS_AT_ONCE; ++u) {
+      const int r = r0 + 4 * u;
+      const unsigned at_slot = unsigned(r * 256 + 4 * chunk) * 4;
 #pragma unroll
-    for (int j = 1; j < GMM_SPLIT_MAX; ++j)
-      if (j < nparts) { acc.x += part[j].x; acc.y += part[j].y; acc.z += part[j].z; acc.w += part[j].w; }
-    const float f[4] = {acc.x, acc.y, acc.z, acc.w};
-    const size_t at = size_t(m0 + r) * ldc + col;
-    if constexpr (OUT_F32) {
-      float* out = reinterpret_cast<float*>(c_group) + at;
-      if (valid == 15) *reinterpret_cast<float4*>(out) = acc;
-      else
+      for (int j = 0; j < GMM_SPLIT_MAX; ++j)
+        if (j < nparts && r < r_end) part[u][j] = gmm_load_device_scope(slots, unsigned(j * tail) * unsigned(GMM_WS_SLOT) + at_slot);
+    }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) if (valid & (1 << e)) out[e] = f[e];
-    } else {
-      uint16_t h[4];
+    for (int u = 0; u < ROWS_AT_ONCE; ++u) {
+      const int r = r0 + 4 * u;
+      if (r >= r_end) break;
+      float4 acc = part[u][0];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if constexpr (F16) { const _Float16 x = _Float16(f[e]); h[e] = *reinterpret_cast<const uint16_t*>(&x); }
-        else h[e] = gmm_bf16_bits(f[e]);
+      for (int j = 1; j < GMM_SPLIT_MAX; ++j)
+        if (j < nparts) { acc.x += part[u][j].x; acc.y += part[u][j].y; acc.z += part[u][j].z; acc.w += part[u][j].w; }
+      const float f[4] = {acc.x, acc.y, acc.z, acc.w};
+      const size_t at = size_t(m0 + r) * ldc + col;
+      if constexpr (OUT_F32) {
+        float* out = reinterpret_cast<float*>(c_group) + at;
+        if (valid == 15) *reinterpret_cast<float4*>(out) = acc;
+        else
+#pragma unroll
+          for (int e = 0; e < 4; ++e) if (valid & (1 << e)) out[e] = f[e];
+      } else {
+        uint16_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (F16) { const _Float16 x = _Float16(f[e]); h[e] = *reinterpret_cast<const uint16_t*>(&x); }
+          else h[e] = gmm_bf16_bits(f[e]);
+        }
+        uint16_t* out = reinterpret_cast<uint16_t*>(c_group) + at;
+        if (valid == 15) *reinterpret_cast<uint2*>(out) = make_uint2(h[0] | (uint32_t(h[1]) << 16), h[2] | (uint32_t(h[3]) << 16));
+        else
+#pragma unroll
+          for (int e = 0; e < 4; ++e) if (valid & (1 << e)) out[e] = h[e];
       }
-      uint16_t* out = reinterpret_cast<uint16_t*>(c_group) + at;
-      if (valid == 15) *reinterpret_cast<uint2*>(out) = make_uint2(h[0] | (uint32_t(h[1]) << 16), h[2] | (uint32_t(h[3]) << 16));
-      else
-#pragma unroll
-        for (int e = 0; e < 4; ++e) if (valid & (1 << e)) out[e] = h[e];
     }
   }
 }
@@ -602,11 +614,12 @@ int gmm_launch_mfma(GmmParams p, GmmLayout lay, int in_dtype, int out_dtype, int
     const int64_t bound = gmm_tile_bound(p.jag, p.G, p.M, p.N, config == GMM_CFG_ASM_256x256 ? p.tall : 256, 256);
     const int64_t want = ((bound + 7) / 8) * 8;
     p.num_wg = int(want < num_cus ? (want < 8 ? 8 : want) : num_cus);
-    // a launch of few tiles with a long contraction can be cut along K to fill the chip
+    // the tiles of a partly filled last round can be cut along K (gmm_tail_split); a launch of few tiles with a
+    // long contraction gets the whole chip for that
     const bool can_split = config == GMM_CFG_ASM_256x256 && p.ws_parts > 0 && !p.act && p.jag != GMM_JAG_K &&
-                           p.K >= 2 * GMM_SPLIT_PART_NK * GMM_TILE_K;
-    if (can_split) p.num_wg = num_cus;
-    else p.ws_parts = 0;
+                           p.K >= 2 * GMM_SPLIT_PART_MIN * GMM_TILE_K;
+    if (can_split && p.K >= 96 * GMM_TILE_K) p.num_wg = num_cus;
+    if (!can_split) p.ws_parts = 0;
   }
   const bool out16 = out_dtype == in_dtype;   // else fp32
   if (!out16 && out_dtype != GMM_DT_F32) return -1;

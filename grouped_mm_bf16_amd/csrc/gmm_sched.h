@@ -65,8 +65,9 @@ struct GmmParams {
 constexpr int GMM_WS_HEADER = 4096;          // 1024 int32: arrival counters, one per tile of the split round, ...
 constexpr int GMM_WS_SLOT = 256 * 256 * 4;   // one fp32 partial tile
 constexpr int GMM_SPLIT_MAX = 8;             // most parts a tile is cut into
-constexpr int GMM_SPLIT_PART_NK = 48;        // K tiles (of 64) a part aims at: long enough to carry its extra fp32
-                                             // store and the reduction, short enough to even out the tail
+constexpr int GMM_SPLIT_PART_MIN = 32;       // fewest K tiles (of 64) of a part
+constexpr int GMM_SPLIT_PART_COST = 20;      // what a part costs beyond its K tiles, in K tiles (gmm_tail_split):
+                                             // measured, a round of 56 tiles of 64 K tiles cut four ways takes as long as uncut
 constexpr int GMM_WS_TICKET = 1020;          // header words beyond the arrival counters: next part to hand out,
 constexpr int GMM_WS_EXITED = 1021;          // workgroups that have left the ticket loop
 
@@ -79,17 +80,22 @@ GMM_HD int gmm_max(int a, int b) { return a > b ? a : b; }
 // every tile of that round is cut along K into S parts (its K tiles split evenly) that any free workgroup
 // takes from a ticket counter; each part stores an fp32 partial tile, and the part that arrives last adds the
 // partials in part order (the sum does not depend on timing) and stores the output.  Returns S (1: no
-// split): parts of about GMM_SPLIT_PART_NK K tiles, at most GMM_SPLIT_MAX per tile, as the workspace allows;
-// no split when the contraction is short or the round is more than three quarters full (the parts' extra
-// stores and the reduction then cost what the idle workgroups would).  nk = K tiles per tile (the same for
-// every tile: not for a jagged contraction).
+// split): the S that makes the round shortest when a part costs its K tiles plus GMM_SPLIT_PART_COST (its
+// prologue, the fp32 store of the partial tile and its share of the reduction, in K tiles) and tail * S parts
+// take ceil(tail * S / W) turns; at most GMM_SPLIT_MAX parts per tile, as the workspace allows, none shorter
+// than GMM_SPLIT_PART_MIN K tiles, and only if the round gets at least a fifth shorter.  nk = K tiles per tile
+// (the same for every tile: not for a jagged contraction).
 GMM_HD int gmm_tail_split(int total, int W, int nk, int max_parts) {
   const int tail = total % W;
-  if (tail == 0 || tail > GMM_WS_TICKET || 4 * tail > 3 * W || nk < 2 * GMM_SPLIT_PART_NK) return 1;
-  int S = (nk + GMM_SPLIT_PART_NK / 2) / GMM_SPLIT_PART_NK;
-  S = gmm_min(S, GMM_SPLIT_MAX);
-  S = gmm_min(S, max_parts / tail);
-  return S < 2 ? 1 : S;
+  if (tail == 0 || tail > GMM_WS_TICKET) return 1;
+  int best = 1, best_cost = nk * 16;                          // costs in sixteenths of a K tile
+  for (int S = 2; S <= GMM_SPLIT_MAX; ++S) {
+    if (S * tail > max_parts || nk / S < GMM_SPLIT_PART_MIN) break;
+    const int turns = (tail * S + W - 1) / W;
+    const int cost = turns * ((nk * 16 + S - 1) / S + GMM_SPLIT_PART_COST * 16);
+    if (cost < best_cost) { best = S; best_cost = cost; }
+  }
+  return (best > 1 && best_cost * 5 <= nk * 16 * 4) ? best : 1;
 }
 
 // K tiles [first, last) of part `part` of S of a tile with nk K tiles.

@@ -254,31 +254,39 @@ def k_coverage(rec, K):
 MIXTRAL = [4812, 1663, 1610, 1663, 1656, 1682, 1633, 1665]
 
 
-def test_down_projection_tail_is_cut_five_ways():
+def test_down_projection_tail_is_cut_four_ways():
     """16384 x 14336 -> 4096 on 256 workgroups: 1008 tall + 80 remainder tiles = 4 rounds + 64 tiles; the 64
-    tiles of the fifth round become 320 parts of 44 or 45 K tiles each."""
+    tiles of the fifth round become 256 parts of 56 K tiles each: one part per workgroup (five parts each would
+    be 320, a second turn for 64 of them)."""
     whole = tile_list3(MIXTRAL, ROWS, 16384, 4096, 14336, 256, 64, 0)
     assert len(whole) == 1088 and (whole[:, 11] == 1).all()
     rec = tile_list3(MIXTRAL, ROWS, 16384, 4096, 14336, 256, 64, 512)
-    assert len(rec) == 1024 + 5 * 64
+    assert len(rec) == 1024 + 4 * 64
     by_tile, n_split = k_coverage(rec, 14336)
     assert len(by_tile) == 1088 and n_split == 64
-    assert (rec[:1024, 11] == 1).all() and (rec[1024:, 11] == 5).all()
+    assert (rec[:1024, 11] == 1).all() and (rec[1024:, 11] == 4).all()
     # without the K ranges the list is the unsplit one: same tiles, same owners
     assert (coverage2(whole[:, :10], 8, 16384, 4096, False) == 1).all()
     first_parts = rec[rec[:, 10] == 0][:, :10]
     assert (coverage2(first_parts, 8, 16384, 4096, False) == 1).all()
     # the parts come in ticket order: K part 0 of every tile of the round, then K part 1, ...
-    assert (rec[1024:, 10] == np.repeat(np.arange(5), 64)).all()
-    # a workspace too small for five parts per tile allows fewer
+    assert (rec[1024:, 10] == np.repeat(np.arange(4), 64)).all()
+    # a workspace too small for four parts per tile allows fewer
     rec = tile_list3(MIXTRAL, ROWS, 16384, 4096, 14336, 256, 64, 128)
     assert len(rec) == 1024 + 2 * 64
 
 
 def test_up_projection_is_left_alone():
-    """16384 x 4096 -> 14336: the last round holds 224 of 256 tiles; cutting them would cost more than it saves."""
+    """16384 x 4096 -> 14336: the last round holds 224 of 256 tiles; cutting them would cost more than it saves.
+    Nor is a thinly filled last round of tiles with 64 K tiles cut: a part costs about 20 K tiles beyond its own
+    (measured: 56 such tiles cut four ways take as long as uncut)."""
     rec = tile_list3(MIXTRAL, ROWS, 16384, 14336, 4096, 256, 64, 512)
     assert len(rec) == 3808 and (rec[:, 11] == 1).all()
+    sizes = [256 * r for r in (20, 7, 6, 6, 6, 7, 6, 7)]          # 65 tile rows: 14 rounds + 56 tiles
+    rec = tile_list3(sizes, ROWS, sum(sizes), 14336, 4096, 256, 64, 512)
+    assert len(rec) == 65 * 56 and (rec[:, 11] == 1).all()
+    rec = tile_list3(sizes, ROWS, sum(sizes), 14336, 8192, 256, 64, 512)   # twice the contraction: cut four ways
+    assert len(rec) == 64 * 56 + 4 * 56 and set(rec[:, 11].tolist()) == {1, 4}
 
 
 @pytest.mark.parametrize("jag,sizes,M,N", [(ROWS, [300, 0, 1, 255, 256, 257, 33], 1102, 700), (COLS, [129, 128, 127, 700], 330, 1084),

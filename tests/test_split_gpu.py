@@ -180,5 +180,5 @@ def test_down_projection_full_size(golden_dir):
         out3 = grouped_mm(ad, bd, offs=offs.to(DEV))
     oracle.assert_close(out3.cpu(), got, 14336)
     if torch.cuda.get_device_properties(0).multi_processor_count == 256:
-        assert n_parts_expected(sizes, 1, 16384, 4096, 14336) == 320
+        assert n_parts_expected(sizes, 1, 16384, 4096, 14336) == 256
         assert not torch.equal(out3.view(torch.int16), out.view(torch.int16))
