@@ -182,9 +182,11 @@ GMM_HD int gmm_find_group(const int32_t* cum, int G, int t) {
 // Skewed group sizes leave many groups far smaller than a tall tile.  The row range of a group is cut
 // into tall tiles; a remainder that fits one shorter tile (64 rows, or 128 under 256-row tall tiles)
 // becomes one: it streams B at the same rate but wastes less MFMA work on rows that do not exist.  A
-// shorter tile runs slower per row (a 128-row tile costs about 0.6, a 64-row tile about 0.35 of a 256-row
-// one), so a remainder that needs two of them pays for another tall tile instead.  All tall tiles of
-// all groups come first in the tile order, the remainder tiles fill the tail of the launch.
+// shorter tile runs slower per row (measured: a 128-row tile costs about 0.76 of a 256-row one -- half the
+// MFMAs for three quarters of the copies per K tile -- and a 64-row tile little less, both being bound by the
+// stream of their B panel), so a remainder that needs two of them pays for another tall tile instead.
+// All tall tiles of all groups come first in the tile order, the remainder tiles fill the tail of the
+// launch (or, group_major, every group's remainder tile follows its tall tiles).
 // `rem_rows` is the height of the group's remainder tile (n_short is 0 or 1).
 GMM_HD void gmm_split_rows(int rows, int tall, int shrt, int& n_tall, int& n_short, int& rem_rows) {
   rem_rows = shrt;
