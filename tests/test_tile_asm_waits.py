@@ -5,7 +5,11 @@ LDS reads complete in the order they were issued, and the generator puts in fron
 variant instruction by instruction with that rule -- a read is known complete only once a wait has left fewer
 reads outstanding than were issued after it -- and fails if an MFMA could issue while one of its operand
 registers is still the destination of a read in flight, or if a read overwrites a fragment register that a
-later MFMA of the same step still wants with its old value."""
+later MFMA of the same step still wants with its old value.
+
+Vector-memory operations (the global -> LDS copies and the prefetch touches) leave their counter in issue order
+too; a second replay follows the prologue and the K loop through whole tiles of 1 to 13 K tiles and fails if a
+barrier that releases a buffer to the fragment reads could be passed while a copy into that buffer is in flight."""
 import importlib.util
 import os
 import re
@@ -136,3 +140,82 @@ def test_the_checker_catches_a_missing_wait():
         for ins in pro[first[0]:] + bodies[(0, True)]:
             if not ins.startswith("s_waitcnt"):
                 lds.step(ins)
+
+
+class Vmem:
+    """Vector-memory operations leave the counter in the order they were issued: `s_waitcnt vmcnt(n)` proves
+    everything but the n youngest complete.  Tracks, for the copies (global -> LDS) in flight, the buffer each
+    one fills: m0 is set to (wave base of A in s76 / of B in s77) + offset right before a copy."""
+
+    def __init__(self, v):
+        self.v = v
+        self.flight = []          # oldest first: buffer index of a copy, None for a touch
+        self.m0 = None
+
+    def step(self, ins):
+        op, _, rest = ins.partition(" ")
+        if op == "s_add_u32" and rest.startswith("m0,"):
+            base, off = [a.strip() for a in rest.split(",")][1:]
+            is_a = base == "s%d" % (gen.S_T + 20)
+            assert is_a or base == "s%d" % (gen.S_T + 21), ins
+            stage = self.v.a_stage if is_a else self.v.b_stage
+            self.m0 = (int(off) - (0 if is_a else self.v.b_base)) // stage
+            assert 0 <= self.m0 < self.v.stages, ins
+        elif op == "buffer_load_dwordx4":
+            assert rest.rstrip().endswith("lds") or " lds" in rest, ins
+            assert self.m0 is not None, "copy without a destination: " + ins
+            self.flight.append(self.m0)
+            self.m0 = None
+        elif op.startswith("buffer_load"):
+            self.flight.append(None)
+        elif op == "s_waitcnt":
+            m = re.search(r"vmcnt\((\d+)\)", rest)
+            if m:
+                keep = int(m.group(1))
+                self.flight = self.flight[len(self.flight) - keep:] if keep else []
+
+    def filling(self):
+        return {b for b in self.flight if b is not None}
+
+
+@pytest.mark.parametrize("a_tr,b_tr,tm", VARIANTS)
+@pytest.mark.parametrize("nk", [1, 2, 3, 4, 5, 8, 13])
+def test_a_k_tile_has_landed_before_its_buffer_is_read(a_tr, b_tr, tm, nk):
+    """Replay of the prologue and of nk K tiles (the interior body where the generated branch takes it): at the
+    barrier that ends the prologue no copy into buffer 0 may be in flight, and at the barrier inside K tile kt
+    none into the buffer of K tile kt + 1 -- the fragment reads that follow each barrier take what is there."""
+    v = gen.Variant(a_tr, b_tr, 0, tm)
+    pro, bodies = loop_bodies(v)
+    S = v.stages
+    vm = Vmem(v)
+    first_barrier = pro.index("s_barrier")
+    for ins in pro[:first_barrier]:
+        vm.step(ins)
+    assert 0 not in vm.filling(), "K tile 0 may still be on its way when the prologue's barrier is passed"
+    for ins in pro[first_barrier:]:
+        vm.step(ins)
+    for kt in range(nk):
+        buf = kt % S
+        interior = kt + S < nk - 1          # the branch in front of every body
+        body = bodies[(buf, interior)]
+        barrier = body.index("s_barrier")
+        for ins in body[:barrier]:
+            vm.step(ins)
+        assert (buf + 1) % S not in vm.filling(), f"K tile {kt + 1} may still be on its way at the barrier of K tile {kt}"
+        for ins in body[barrier:]:
+            vm.step(ins)
+
+
+def test_the_copy_checker_catches_a_wait_that_allows_too_much():
+    v = gen.Variant(0, 1, 0, 4)
+    pro, bodies = loop_bodies(v)
+    vm = Vmem(v)
+    for ins in pro:
+        vm.step(ins)
+    body = bodies[(0, True)]
+    barrier = body.index("s_barrier")
+    for ins in body[:barrier]:
+        if ins.startswith("s_waitcnt vmcnt"):
+            ins = re.sub(r"vmcnt\(\d+\)", "vmcnt(%d)" % (v.nt + 1), ins)   # one operation more than the touches
+        vm.step(ins)
+    assert 1 in vm.filling()
