@@ -219,3 +219,65 @@ def test_the_copy_checker_catches_a_wait_that_allows_too_much():
             ins = re.sub(r"vmcnt\(\d+\)", "vmcnt(%d)" % (v.nt + 1), ins)   # one operation more than the touches
         vm.step(ins)
     assert 1 in vm.filling()
+
+
+def read_buffer(v, ins):
+    """(operand, buffer) a fragment read takes its data from, or None for any other instruction."""
+    m = re.match(r"ds_read_b(?:128|64_tr_b16) \S+, v(\d+)(?: offset:(\d+))?", ins)
+    if not m:
+        return None
+    reg, off = int(m.group(1)), int(m.group(2) or 0)
+    if gen.V_TMP <= reg < gen.V_TMP + 12:
+        return None     # the masking of a partial first / last k chunk: its own stretch between two barriers, no copies in it
+    if v.stages == 2:
+        is_a = reg in (gen.V_RA, gen.V_RA + 1)
+        assert is_a or reg in (gen.V_RB, gen.V_RB + 1), ins
+        return ("A" if is_a else "B", off // (v.a_stage if is_a else v.b_stage))
+    is_a = gen.V_BUFA <= reg < gen.V_BUFA + 6
+    assert is_a or gen.V_BUFB <= reg < gen.V_BUFB + 6, ins
+    return ("A" if is_a else "B", (reg - (gen.V_BUFA if is_a else gen.V_BUFB)) // 2)
+
+
+@pytest.mark.parametrize("a_tr,b_tr,tm", VARIANTS)
+def test_no_buffer_is_copied_into_between_the_barriers_that_it_is_read_between(a_tr, b_tr, tm):
+    """The four waves of a workgroup run the same code and meet at every barrier, so what one wave reads and what
+    another one overwrites can only collide inside one stretch between two barriers: there, the buffers read and
+    the buffers that copies are aimed at must differ."""
+    v = gen.Variant(a_tr, b_tr, 0, tm)
+    pro, bodies = loop_bodies(v)
+    S = v.stages
+    for nk in (1, 2, 3, 5, 9):
+        stream = list(pro)
+        for kt in range(nk):
+            stream += bodies[(kt % S, kt + S < nk - 1)]
+        check_stretches(v, stream)
+
+
+def check_stretches(v, stream):
+    read, written, m0 = set(), set(), None
+    for ins in stream:
+        if ins == "s_barrier":
+            read, written = set(), set()
+        elif ins.startswith("s_add_u32 m0,"):
+            base, off = [a.strip() for a in ins.split(" ", 1)[1].split(",")][1:]
+            is_a = base == "s%d" % (gen.S_T + 20)
+            m0 = ("A" if is_a else "B", (int(off) - (0 if is_a else v.b_base)) // (v.a_stage if is_a else v.b_stage))
+        elif ins.startswith("buffer_load_dwordx4"):
+            written.add(m0)
+        elif read_buffer(v, ins):
+            read.add(read_buffer(v, ins))
+        assert not read & written, (ins, sorted(read & written))
+
+
+def test_the_stretch_checker_catches_a_copy_into_the_buffer_being_read():
+    v = gen.Variant(0, 1, 0, 4)
+    pro, bodies = loop_bodies(v)
+    body = list(bodies[(0, True)])
+    # step 3's copies (after the barrier) go into buffer 0; moved in front of the barrier they hit the buffer
+    # that steps 0 to 2 read
+    barrier = body.index("s_barrier")
+    late = [i for i in range(barrier, len(body)) if body[i].startswith("s_add_u32 m0,")][0]
+    moved = body[late:late + 3]
+    assert any(x.startswith("buffer_load_dwordx4") for x in moved)
+    with pytest.raises(AssertionError):
+        check_stretches(v, pro + body[:barrier] + moved + body[barrier:])
