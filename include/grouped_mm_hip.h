@@ -216,8 +216,7 @@ int gmm_last_mfma_config(void);
 int gmm_set_xcd_remap(int on);
 /* Launch order of the assembly tile's kernel: 0 = all tall tiles of all groups, then the remainder tiles;
  * 1 = group by group; -1 (default) = chosen from the shapes (group by group when the tall tiles are 128 rows,
- * the regime of many small groups, and for jagged rows under an output of at least 8192 columns).  Returns the
- * previous setting. */
+ * the regime of many small groups).  Returns the previous setting. */
 int gmm_set_group_major(int mode);
 /* 0: later launches ignore their workspace, so no tile is cut along the contraction (tests compare launches
  * bit for bit that would otherwise split differently); 1 (default): use it.  Returns the previous setting. */
