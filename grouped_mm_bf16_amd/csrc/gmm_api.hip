@@ -155,17 +155,11 @@ int run(Problem& pr, hipStream_t stream) {
       if (lay.a_kc && (fs == 0 || fs == 64)) p.shrt = fs;
     }
     // Launch order: group by group in the fine-grained regime (many small groups: a group's remainder tile
-    // then reads the second operand while its tall tiles have it in the caches; +4 % there), and for jagged rows
-    // under an output at least 32 tiles wide (a group's remainder row then fills whole XCD blocks by itself and
-    // finds the group's second operand in the Infinity Cache instead of fetching it from memory again at the end
-    // of the launch: Mixtral up projection 1.2 % faster).  Otherwise all tall tiles first: a narrower remainder
-    // row shares its XCD blocks with the next group's tall tiles, and workgroups on tiles of different heights
-    // fall out of step (the down projection, 16 tiles wide, loses 0.4 to 1.3 % group by group, the fine-grained
-    // up projection of a mixture-of-experts layer, 6 tiles wide, 5 %).
+    // then reads the second operand while its tall tiles have it in the caches; +4 % there), otherwise all
+    // tall tiles first (longest first balances the rounds; the down projection loses 1 % group by group).
     {
       const int fo = g_group_major.load(std::memory_order_relaxed);
-      const bool wide_rows = p.jag == GMM_JAG_M && p.N >= 32 * 256;   // 256 = width of a tile
-      p.group_major = fo >= 0 ? fo : ((p.tall == 128 || wide_rows) ? 1 : 0);
+      p.group_major = fo >= 0 ? fo : (p.tall == 128 ? 1 : 0);
     }
     rc = gmm_launch_mfma(p, lay, pr.in_dtype, pr.out_dtype, cfg, cus, stream);
     t_last_path = GMM_PATH_MFMA;
